@@ -168,7 +168,8 @@ typedef struct {
  * (test_fused_deep_moe.py:66-69); the equivalent step here is
  * zbal_moe_weight_prepack(), which turns the logical [E, K, N] row-major
  * tensor into ZBAL_WEIGHT_FORMAT_KCONTIG: [E, N, K] with K contiguous
- * (for INT4X2: [E, N, K/2] bytes, low nibble = even k).
+ * (for INT4X2: [E, N, K/2] bytes; in each group of 8 consecutive k, byte b
+ * holds k[b] in the low and k[b+4] in the high nibble).
  */
 #define ZBAL_WEIGHT_FORMAT_ND      0 /* logical [E, K, N], N contiguous */
 #define ZBAL_WEIGHT_FORMAT_KCONTIG 1 /* [E, N, K], K contiguous         */

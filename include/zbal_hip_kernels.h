@@ -1,0 +1,161 @@
+/*
+ * Inner C ABI: the HIP kernel launchers the zbal operator layer sits on.
+ *
+ * This is the seam the reference calls "zbal_kernel": its host launchers
+ * ZBALOp* (app/zbal/src/csrc/operators/npu/zbal_npu_operators.h:18-97) take
+ * tensor descriptors and a CommGroupInfo; the functions below take the same
+ * information as plain device pointers and sizes so that C, ctypes, cgo or
+ * JNI callers can drive the kernels without the communicator layer.
+ *
+ * Conventions: every pointer is a device pointer unless stated; `stream` is
+ * a hipStream_t passed as void* (NULL = null stream); launches are
+ * asynchronous; the return value is 0 or a negative ZResult (-2 invalid
+ * parameter, -11 HIP runtime error). One rank (R = 1) owns all `experts`;
+ * rows of the permuted activation matrix are expert-major in flat (t,k)
+ * pick order. dtype arguments are zbal_datatype_t values.
+ */
+#ifndef ZBAL_HIP_KERNELS_H_
+#define ZBAL_HIP_KERNELS_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* exported even when the library is built with hidden default visibility */
+#define ZBALHIP_API __attribute__((visibility("default")))
+
+#define ZBALHIP_MAX_REDUCE_PEERS 16
+#define ZBALHIP_LAYOUT_MAX_BLOCKS 50 /* scratch rows, reference dispatch_layout.h:33 (MAX_BLOCK) */
+
+/*
+ * Router (no reference counterpart). logits [T,E] fp32 -> topk_idx [T,K]
+ * int64, topk_w [T,K] fp32. E <= 1024, K <= 32, K <= E.
+ */
+ZBALHIP_API int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64_t experts, int64_t topk, int64_t *topk_idx,
+                           float *topk_w, void *stream);
+
+/*
+ * Replaces ZBALOpDispatchLayout (zbal_npu_operators.h:47-50; kernel
+ * dispatch_layout.h:97-183). idx_is_i64 selects int64 or int32 indices.
+ * Outputs: tokens_per_rank [ranks] i32, tokens_per_expert [experts] i32,
+ * send_token_idx [T,K] i32 (-1 for picks outside [0,experts)).
+ * scratch: [ZBALHIP_LAYOUT_MAX_BLOCKS * experts] i32, contents undefined after.
+ */
+ZBALHIP_API int32_t zbalhip_dispatch_layout(const void *topk_idx, int32_t idx_is_i64, int64_t tokens, int64_t experts, int64_t topk,
+                                int32_t ranks, int32_t *tokens_per_rank, int32_t *tokens_per_expert,
+                                int32_t *send_token_idx, int32_t *scratch, void *stream);
+
+/*
+ * Replaces ZBALOpNotifyDispatch (zbal_npu_operators.h:52-56; kernel
+ * notify_dispatch.h:356-596) for one rank: recv_data [1,E] = counts,
+ * put_offset [E] = exclusive cumsum, total_recv [1], recv_tokens_per_expert
+ * [E] i64, balance_matrix [1,2] = {0, tokens-1} (or {-1,-1} when no pick).
+ */
+ZBALHIP_API int32_t zbalhip_dispatch_notify(const int32_t *tokens_per_expert, int64_t experts, int64_t topk, int32_t *recv_data,
+                                int32_t *put_offset, int32_t *total_recv, int64_t *recv_tokens_per_expert,
+                                int32_t *balance_matrix, void *stream);
+
+/*
+ * Replaces ZBALOpDispatchNormal (zbal_npu_operators.h:58-62; kernel
+ * dispatch_normal.h:479-563). quant_mode: 0 copy, 1 int8 per token with
+ * s = 127/(amax+1e-12), 2 e4m3 with 1x128 scales (dest_scale [rows, H/128]).
+ * x_dtype: BFP16 or FP16. hidden % 16 == 0 (mode 2: % 128 == 0).
+ */
+ZBALHIP_API int32_t zbalhip_dispatch_normal(const void *x, int32_t x_dtype, const int32_t *topk_idx, const int32_t *send_token_idx,
+                                const int32_t *put_offset, int64_t tokens, int64_t hidden, int64_t topk,
+                                int64_t experts, int32_t quant_mode, void *dest, float *dest_scale, void *stream);
+
+/*
+ * Replaces ZBALOpCombineNormal (zbal_npu_operators.h:64-68; kernel
+ * combine_normal.h:398-494): out[t] = round(sum_k fp32(y[base[e]+idx]) * w),
+ * multiply and add rounded separately, k ascending, invalid ids skipped.
+ * base_is_inclusive = 1 reads `base` as the low-latency kernels' inclusive
+ * running counts (combine_low_latency.h:504-506).
+ */
+ZBALHIP_API int32_t zbalhip_combine(const void *y, int32_t dtype, const int32_t *base, int32_t base_is_inclusive, const float *w,
+                        const int32_t *topk_idx, const int32_t *send_token_idx, int64_t tokens, int64_t hidden,
+                        int64_t topk, int64_t experts, void *out, void *stream);
+
+/*
+ * Replaces ZBALOpDispatchLowLatency (zbal_npu_operators.h:70-77; kernel
+ * dispatch_low_latency.h:528-844) for one rank: layout, counts and the
+ * quantising permute in one call. quant_mode 1 uses s = 127/amax (an
+ * all-zero row gives q = 0, scale = 0). ep_recv_counts [E] = inclusive
+ * running sum; expert_token_nums [E] i64 = counts (type 1) or the running
+ * sum (type 0). scratch holds scratch_blocks * experts i32 (scratch_blocks
+ * >= 1 bounds the number of workgroups of the layout pass).
+ */
+ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, const int32_t *expert_ids, int64_t tokens,
+                                     int64_t hidden, int64_t topk, int64_t experts, int32_t quant_mode,
+                                     int32_t token_nums_type, void *expand_x, float *dynamic_scales,
+                                     int32_t *expand_idx, int64_t *expert_token_nums, int32_t *ep_recv_counts,
+                                     int32_t *scratch, int32_t scratch_blocks, void *stream);
+
+/*
+ * The local reduction under ZBALOpReduceScatter / ZBALOpAllReduce
+ * (zbal_npu_operators.h:21-25; kernels reducescatter.cpp:94-151,
+ * allreduce.cpp:206-260): out[j] = op over p = 0..n_in-1 of in[p][j].
+ * `in` is a HOST array of n_in <= ZBALHIP_MAX_REDUCE_PEERS device pointers.
+ * Float types accumulate in fp32 in order p = 0..n_in-1 and round once.
+ * op is a zbal_reduce_op_t value; PROD is a true product.
+ */
+ZBALHIP_API int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t count, int32_t dtype, int32_t op, void *out,
+                       void *stream);
+
+/*
+ * Weight pre-pack: [E,K,N] (N contiguous) -> [E,N,K] (K contiguous);
+ * to_int4 != 0 packs int8 values in [-8,7] two per byte ([E,N,K/2]).
+ */
+ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int64_t k, int64_t n, int32_t to_int4, void *dst,
+                               void *stream);
+
+/*
+ * Permute + quantise stage of the fused operator (QuantToken /
+ * LocalQuantFunc, FDM/gemm/kernel/…swiglu_quant_multistage_workspace.h:
+ * 952-995, 1859-2058). mode 1: int8, s = 127/amax, optional smooth [E,H]
+ * fp32 multiplied in first; mode 2: e4m3 1x128. Outputs q1 [rows,H], xs
+ * ([rows] or [rows,H/128]), expand_idx [T,K], counts [E] i64 and the
+ * exclusive row offsets row_off [E+1] i32. scratch / scratch_blocks as above.
+ */
+ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids, const float *smooth,
+                                    int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int32_t mode,
+                                    void *q1, float *xs, int32_t *expand_idx, int64_t *counts, int32_t *row_off,
+                                    int32_t *scratch, int32_t scratch_blocks, void *stream);
+
+/*
+ * Grouped GEMM 1 with dequant + SwiGLU + requant epilogue (AIC loop
+ * …swiglu_quant_multistage_workspace.h:603-833, epilogue
+ * block_epilogue_per_token_dequant_swiglu.h:171-298, BlockQuant
+ * …workspace.h:87-316). a [rows,K] expert-major; w1 pre-packed [E,N1,K];
+ * row_off [E+1] exclusive offsets (device). mode 1 (W8A8): w1scale fp32
+ * [E,N1]; q2 int8 [rows,N1/2], scale2 [rows]; sgl_ws is scratch of
+ * max_rows * (N1/2 + 1) * 4 bytes (fp32 SwiGLU values, then one row maximum
+ * each). mode 2 (fp8): a_scale [rows,K/128], w1scale fp32
+ * [E,K/128,N1/128]; q2 e4m3, scale2 [rows,N1/256]; sgl_ws unused.
+ * mode 3 (W4A8): w1 int4x2 [E,N1,K/2], w1scale fp16 [E,K/128,N1];
+ * outputs as mode 1. max_rows bounds the launch (>= total rows).
+ */
+ZBALHIP_API int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale, const void *w1, const void *w1scale,
+                                  const int32_t *row_off, int64_t experts, int64_t max_rows, int64_t k, int64_t n1,
+                                  int32_t mode, void *q2, float *scale2, float *sgl_ws, void *stream);
+
+/*
+ * Grouped GEMM 2 with dequant epilogue (kernel
+ * grouped_matmul_slice_m_per_token_dequant_multistage_workspace.h:166-548,
+ * epilogue block_epilogue_per_token_dequant.hpp:265-397):
+ * y[m,n] = round((float(C) * wscale[g,n]) * a_scale[m]) for mode 1
+ * (wscale_dtype FP32 or BFP16, [E,N]); block-scaled for mode 2
+ * (wscale fp32 [E,K/128,N/128], a_scale [rows,K/128]); group-scaled for
+ * mode 3 (wscale fp16 [E,K/128,N]). w2 pre-packed [E,N,K]. y dtype BFP16/FP16.
+ */
+ZBALHIP_API int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, const void *w2, const void *wscale,
+                             int32_t wscale_dtype, const int32_t *row_off, int64_t experts, int64_t max_rows,
+                             int64_t k, int64_t n, int32_t mode, int32_t out_dtype, void *y, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* ZBAL_HIP_KERNELS_H_ */

@@ -141,7 +141,7 @@ int32_t zbal_moe_topk_route(const zbal_tensor_info_t *logits, int64_t topkNum, c
  * ([E, K, N], N contiguous, one byte per element) to
  * ZBAL_WEIGHT_FORMAT_KCONTIG ([E, N, K]). When dst->dataType is INT4X2 the
  * source is INT8 with values in [-8, 7] and the result packs two of them per
- * byte ([E, N, K/2], low nibble = even k). `dst` must not alias `src`. The
+ * byte ([E, N, K/2]; nibble order as documented for ZBAL_WEIGHT_FORMAT_KCONTIG). `dst` must not alias `src`. The
  * stand-in for the reference's format cast of fused-kernel weights
  * (test_fused_deep_moe.py:66-69).
  */

@@ -1,0 +1,529 @@
+/*
+ * HIP backend of the communicator: checks tensor descriptors against what
+ * each kernel assumes (type, rank, extent, alignment), then forwards to the
+ * zbalhip_* launchers. The counterpart of the reference's
+ * operators/npu/zbal_npu_communicator_base.cpp, which forwards each virtual
+ * to a ZBALOp* launcher (:306-369 for the MoE operators, :371-438 for the
+ * fused one).
+ *
+ * MoE operators run for a group of one rank: the rank owns all experts and
+ * "peer" output buffers are the caller's local tensors. Reductions run over
+ * the group's registered peer windows.
+ */
+#include <cstring>
+
+#include "zbal_hip_kernels.h"
+#include "zbal_host.h"
+
+namespace zbal {
+
+namespace {
+
+int64_t Numel(const zbal_tensor_info_t *t)
+{
+    if (t->dim == 0 || t->dim > ZBAL_MAX_TENSOR_DIM) return 0;
+    int64_t n = 1;
+    for (int i = 0; i < t->dim; ++i) n *= t->shape[i];
+    return n;
+}
+
+const char *DtName(int dt)
+{
+    static const char *names[] = {"int8",  "int16", "int32",  "int64",  "uint64", "fp64",    "fp16",
+                                  "fp32",  "bf16",  "uint8",  "uint16", "uint32", "fp8e4m3", "int4x2"};
+    return (dt >= 0 && dt < ZBAL_DATA_TYPE_BUTT) ? names[dt] : "?";
+}
+
+/* data non-null, one of two allowed types, at least min_elems elements */
+bool CheckTensor(const char *op, const char *name, const zbal_tensor_info_t *t, int dt_a, int dt_b, int64_t min_elems)
+{
+    if (t->data == nullptr) {
+        ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as " << name << " has no data");
+        return false;
+    }
+    if ((int)t->dataType != dt_a && (int)t->dataType != dt_b) {
+        ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as " << name << " has type " << DtName(t->dataType) << ", expected "
+                                       << DtName(dt_a) << (dt_b != dt_a ? std::string(" or ") + DtName(dt_b) : ""));
+        return false;
+    }
+    if (Numel(t) < min_elems) {
+        ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as " << name << " holds " << Numel(t) << " elements, needs "
+                                       << min_elems);
+        return false;
+    }
+    if ((reinterpret_cast<uintptr_t>(t->data) & 15u) != 0) {
+        ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as " << name << " is not 16-byte aligned");
+        return false;
+    }
+    return true;
+}
+
+#define ZB_CHECK(...)                           \
+    do {                                        \
+        if (!CheckTensor(__VA_ARGS__)) return Z_INVALID_PARAM; \
+    } while (0)
+
+int32_t Launched(const char *op, int32_t rc)
+{
+    if (rc != 0) ZBAL_LOG_AND_SET_LAST_ERROR(op << " launch failed, code " << rc);
+    return rc;
+}
+
+class GpuCommunicator final : public Communicator {
+public:
+    using Communicator::Communicator;
+
+    bool SingleRank(const char *op) const
+    {
+        if (info_.groupSize == 1) return true;
+        ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as this build runs MoE operators on a group of one rank, group has "
+                                       << info_.groupSize);
+        return false;
+    }
+
+    /* address of `p` (inside my window) in rank r's window */
+    bool Translate(const char *op, const void *p, size_t bytes, const void **out) const
+    {
+        const PeerWindow &mine = info_.peers[info_.myGroupRank];
+        const uintptr_t a = reinterpret_cast<uintptr_t>(p), b = reinterpret_cast<uintptr_t>(mine.base);
+        if (mine.base == nullptr || a < b || a + bytes > b + mine.size) {
+            ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as the send buffer is not inside this rank's registered window");
+            return false;
+        }
+        for (uint16_t r = 0; r < info_.groupSize; ++r) {
+            const PeerWindow &w = info_.peers[r];
+            if (w.base == nullptr || (a - b) + bytes > w.size) {
+                ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as rank " << r << " has no window covering the buffer");
+                return false;
+            }
+            out[r] = static_cast<const uint8_t *>(w.base) + (a - b);
+        }
+        return true;
+    }
+
+    static size_t ElemSize(zbal_datatype_t dt)
+    {
+        switch (dt) {
+            case ZBAL_DATA_TYPE_INT8: case ZBAL_DATA_TYPE_UINT8: return 1;
+            case ZBAL_DATA_TYPE_INT16: case ZBAL_DATA_TYPE_UINT16: case ZBAL_DATA_TYPE_FP16: case ZBAL_DATA_TYPE_BFP16: return 2;
+            case ZBAL_DATA_TYPE_INT32: case ZBAL_DATA_TYPE_UINT32: case ZBAL_DATA_TYPE_FP32: return 4;
+            case ZBAL_DATA_TYPE_INT64: case ZBAL_DATA_TYPE_UINT64: case ZBAL_DATA_TYPE_FP64: return 8;
+            default: return 0;
+        }
+    }
+
+    int32_t Reduce(const char *opName, const void *send, size_t sliceOffsetElems, void *recv, size_t count,
+                   zbal_datatype_t dt, zbal_reduce_op_t op, aclrtStream stream)
+    {
+        switch (dt) { /* the types the reference instantiates, zbal_kernel_allreduce.cpp:378-416 */
+            case ZBAL_DATA_TYPE_INT8: case ZBAL_DATA_TYPE_INT16: case ZBAL_DATA_TYPE_INT32: case ZBAL_DATA_TYPE_INT64:
+            case ZBAL_DATA_TYPE_FP16: case ZBAL_DATA_TYPE_BFP16: case ZBAL_DATA_TYPE_FP32: break;
+            default:
+                ZBAL_LOG_AND_SET_LAST_ERROR(opName << " failed as data type " << DtName(dt) << " is not supported");
+                return Z_INVALID_PARAM;
+        }
+        if (info_.groupSize > ZBALHIP_MAX_REDUCE_PEERS) {
+            ZBAL_LOG_AND_SET_LAST_ERROR(opName << " failed as group size " << info_.groupSize << " exceeds "
+                                               << ZBALHIP_MAX_REDUCE_PEERS);
+            return Z_INVALID_PARAM;
+        }
+        const size_t es = ElemSize(dt);
+        const void *peer[ZBALHIP_MAX_REDUCE_PEERS];
+        if (info_.groupSize == 1 && info_.peers[0].base == nullptr) {
+            peer[0] = send; /* a group of one needs no window */
+        } else if (!Translate(opName, send, (sliceOffsetElems + count) * es, peer)) {
+            return Z_INVALID_PARAM;
+        }
+        for (uint16_t r = 0; r < info_.groupSize; ++r)
+            peer[r] = static_cast<const uint8_t *>(peer[r]) + sliceOffsetElems * es;
+        return Launched(opName, zbalhip_reduce(peer, info_.groupSize, (int64_t)count, dt, op, recv, stream));
+    }
+
+    int32_t AllReduce(const void *send, void *recv, void *, size_t count, zbal_datatype_t dt, zbal_reduce_op_t op,
+                      aclrtStream stream) override
+    {
+        return Reduce("AllReduce", send, 0, recv, count, dt, op, stream);
+    }
+
+    int32_t ReduceScatter(const void *send, void *recv, size_t recvCount, zbal_datatype_t dt, zbal_reduce_op_t op,
+                          aclrtStream stream) override
+    {
+        return Reduce("ReduceScatter", send, (size_t)info_.myGroupRank * recvCount, recv, recvCount, dt, op, stream);
+    }
+
+    int32_t DispatchNormalLayout(const zbal_tensor_info_t *topkIndex, int64_t tokens, int64_t expertNum,
+                                 int64_t topkNum, const zbal_tensor_info_t *tokensPerRank,
+                                 const zbal_tensor_info_t *tokensPerExpert, const zbal_tensor_info_t *sendTokensIndex,
+                                 const zbal_tensor_info_t *notifySendData, aclrtStream stream, int64_t) override
+    {
+        const char *op = "DispatchLayout";
+        const int64_t R = info_.groupSize;
+        ZBAL_VALIDATE_RETURN(expertNum % R == 0, op << " failed as expertNum " << expertNum
+                                                    << " is not a multiple of the group size " << R, Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(expertNum <= 1024, op << " failed as expertNum " << expertNum << " exceeds 1024",
+                             Z_INVALID_PARAM);
+        ZB_CHECK(op, "tokensPerRank", tokensPerRank, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, R);
+        ZB_CHECK(op, "tokensPerExpert", tokensPerExpert, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum);
+        ZB_CHECK(op, "notifySendData", notifySendData, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32,
+                 (int64_t)ZBALHIP_LAYOUT_MAX_BLOCKS * expertNum);
+        if (tokens > 0) {
+            ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT32, tokens * topkNum);
+            ZB_CHECK(op, "sendTokensIndex", sendTokensIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32,
+                     tokens * topkNum);
+        }
+        return Launched(op, zbalhip_dispatch_layout(topkIndex->data, topkIndex->dataType == ZBAL_DATA_TYPE_INT64,
+                                                    tokens, expertNum, topkNum, (int32_t)R,
+                                                    (int32_t *)tokensPerRank->data, (int32_t *)tokensPerExpert->data,
+                                                    (int32_t *)sendTokensIndex->data, (int32_t *)notifySendData->data,
+                                                    stream));
+    }
+
+    int32_t DispatchNormalNotify(const zbal_tensor_info_t *sendTokensPerExpert, int64_t sendCount, int64_t topKNum,
+                                 const zbal_tensor_info_t *recvBuff, const zbal_tensor_info_t *totalRecvTokens,
+                                 const zbal_tensor_info_t *recvTokensPerExpert,
+                                 const zbal_tensor_info_t *pushTargetOffset, const zbal_tensor_info_t *balanceMatrix,
+                                 aclrtStream stream, int64_t) override
+    {
+        const char *op = "NotifyDispatch";
+        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        const int64_t E = sendCount; /* one count per expert, zbal_deepep.cpp:325-326 */
+        ZBAL_VALIDATE_RETURN(E <= 1024, op << " failed as sendCount " << E << " exceeds 1024", Z_INVALID_PARAM);
+        ZB_CHECK(op, "sendTokensPerExpert", sendTokensPerExpert, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        ZB_CHECK(op, "recvBuff", recvBuff, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        ZB_CHECK(op, "totalRecvTokens", totalRecvTokens, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, 1);
+        ZB_CHECK(op, "recvTokensPerExpert", recvTokensPerExpert, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
+        ZB_CHECK(op, "pushTargetOffset", pushTargetOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        ZB_CHECK(op, "balanceMatrix", balanceMatrix, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, 2);
+        return Launched(op, zbalhip_dispatch_notify((const int32_t *)sendTokensPerExpert->data, E, topKNum,
+                                                    (int32_t *)recvBuff->data, (int32_t *)pushTargetOffset->data,
+                                                    (int32_t *)totalRecvTokens->data,
+                                                    (int64_t *)recvTokensPerExpert->data,
+                                                    (int32_t *)balanceMatrix->data, stream));
+    }
+
+    static bool TokensShape(const char *op, const zbal_tensor_info_t *x, int64_t *tokens, int64_t *hidden)
+    {
+        if (x->dim != 2) {
+            ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as the token tensor must be [tokens, hidden]");
+            return false;
+        }
+        *tokens = x->shape[0];
+        *hidden = x->shape[1];
+        return true;
+    }
+
+    int32_t DispatchNormal(const zbal_tensor_info_t *srcTokens, const zbal_tensor_info_t *topkIndex,
+                           const zbal_tensor_info_t *sendTokensIndex, const zbal_tensor_info_t *pushTargetOffset,
+                           const zbal_tensor_info_t *, int64_t expertNum, zbal_quant_mode_t quantMode,
+                           const zbal_tensor_info_t *destTokens, const zbal_tensor_info_t *destScale,
+                           aclrtStream stream, int64_t) override
+    {
+        const char *op = "DispatchNormal";
+        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        int64_t T = 0, H = 0;
+        if (!TokensShape(op, srcTokens, &T, &H)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(topkIndex->dim == 2 && topkIndex->shape[0] == T, op << " failed as topkIndex must be [tokens, topk]",
+                             Z_INVALID_PARAM);
+        const int64_t K = topkIndex->shape[1];
+        ZBAL_VALIDATE_RETURN(quantMode == NO_QUANT || quantMode == QUANT_BF16_2_INT8 ||
+                                 quantMode == QUANT_BF16_2_FP8E4M3_B128,
+                             op << " failed as quantMode " << quantMode << " is invalid", Z_INVALID_PARAM);
+        /* rows are stored densely; the reference pads row strides to 32 bytes (dispatch_normal.h:215) */
+        const int64_t rowBytes = H * (quantMode == NO_QUANT ? 2 : 1);
+        ZBAL_VALIDATE_RETURN(rowBytes % 32 == 0, op << " failed as a row of " << rowBytes << " bytes is not a multiple of 32",
+                             Z_INVALID_PARAM);
+        if (T == 0) return Z_OK;
+        ZB_CHECK(op, "srcTokens", srcTokens, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
+        ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "sendTokensIndex", sendTokensIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "pushTargetOffset", pushTargetOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum);
+        if (quantMode == NO_QUANT) {
+            ZB_CHECK(op, "destTokens", destTokens, srcTokens->dataType, srcTokens->dataType, H);
+        } else if (quantMode == QUANT_BF16_2_INT8) {
+            ZB_CHECK(op, "destTokens", destTokens, ZBAL_DATA_TYPE_INT8, ZBAL_DATA_TYPE_INT8, H);
+            ZB_CHECK(op, "destScale", destScale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, 1);
+        } else {
+            ZB_CHECK(op, "destTokens", destTokens, ZBAL_DATA_TYPE_FP8_E4M3, ZBAL_DATA_TYPE_UINT8, H);
+            ZB_CHECK(op, "destScale", destScale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, H / 128);
+        }
+        return Launched(op, zbalhip_dispatch_normal(srcTokens->data, srcTokens->dataType, (const int32_t *)topkIndex->data,
+                                                    (const int32_t *)sendTokensIndex->data,
+                                                    (const int32_t *)pushTargetOffset->data, T, H, K, expertNum,
+                                                    (int32_t)quantMode, destTokens->data, (float *)destScale->data,
+                                                    stream));
+    }
+
+    int32_t CombineNormal(const zbal_tensor_info_t *srcTokens, const zbal_tensor_info_t *srcTokensPerEp,
+                          const zbal_tensor_info_t *topKWeight, const zbal_tensor_info_t *topkIndex,
+                          const zbal_tensor_info_t *sendTokensIndex, const zbal_tensor_info_t *, uint16_t expertNum,
+                          const zbal_tensor_info_t *destTokens, aclrtStream stream, int64_t) override
+    {
+        const char *op = "CombineNormal";
+        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        int64_t T = 0, H = 0;
+        if (!TokensShape(op, destTokens, &T, &H)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(topkIndex->dim == 2 && topkIndex->shape[0] == T, op << " failed as topkIndex must be [tokens, topk]",
+                             Z_INVALID_PARAM);
+        const int64_t K = topkIndex->shape[1];
+        ZBAL_VALIDATE_RETURN(K <= 32, op << " failed as topk " << K << " exceeds 32", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN((H * 2) % 32 == 0, op << " failed as hidden " << H << " gives rows that are not a multiple of 32 bytes",
+                             Z_INVALID_PARAM);
+        if (T == 0) return Z_OK;
+        ZB_CHECK(op, "srcTokens", srcTokens, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, H);
+        ZBAL_VALIDATE_RETURN(srcTokens->dataType == destTokens->dataType, op << " failed as source and destination types differ",
+                             Z_INVALID_PARAM);
+        ZB_CHECK(op, "destTokens", destTokens, srcTokens->dataType, srcTokens->dataType, T * H);
+        ZB_CHECK(op, "srcTokensPerEp", srcTokensPerEp, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum);
+        ZB_CHECK(op, "topKWeight", topKWeight, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
+        ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "sendTokensIndex", sendTokensIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        return Launched(op, zbalhip_combine(srcTokens->data, srcTokens->dataType, (const int32_t *)srcTokensPerEp->data, 0,
+                                            (const float *)topKWeight->data, (const int32_t *)topkIndex->data,
+                                            (const int32_t *)sendTokensIndex->data, T, H, K, expertNum,
+                                            destTokens->data, stream));
+    }
+
+    int32_t DispatchLowLatency(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds, int64_t moeExpertNum,
+                               int64_t, int64_t sharedExpertRankNum, int64_t quantMode, int64_t, int64_t,
+                               int64_t expertTokenNumsType, const zbal_tensor_info_t *expandXOut,
+                               const zbal_tensor_info_t *dynamicScalesOut, const zbal_tensor_info_t *expandIdxOut,
+                               const zbal_tensor_info_t *expertTokenNumsOut, const zbal_tensor_info_t *epRecvCountsOut,
+                               const zbal_tensor_info_t *putOffset, const zbal_tensor_info_t *, aclrtStream stream,
+                               int64_t) override
+    {
+        const char *op = "DispatchLowlatency";
+        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(sharedExpertRankNum == 0, op << " failed as shared expert ranks are not supported", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(expertTokenNumsType == 0 || expertTokenNumsType == 1,
+                             op << " failed as expertTokenNumsType " << expertTokenNumsType << " is invalid", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(quantMode >= 0 && quantMode <= 2, op << " failed as quantMode " << quantMode << " is invalid",
+                             Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(moeExpertNum <= 1024, op << " failed as moeExpertNum exceeds 1024", Z_INVALID_PARAM);
+        int64_t T = 0, H = 0;
+        if (!TokensShape(op, x, &T, &H)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(expertIds->dim == 2 && expertIds->shape[0] == T, op << " failed as expertIds must be [tokens, topk]",
+                             Z_INVALID_PARAM);
+        const int64_t K = expertIds->shape[1];
+        const int64_t rowBytes = H * (quantMode == 0 ? 2 : 1);
+        ZBAL_VALIDATE_RETURN(rowBytes % 32 == 0, op << " failed as a row of " << rowBytes << " bytes is not a multiple of 32",
+                             Z_INVALID_PARAM);
+        const int64_t E = moeExpertNum;
+        ZB_CHECK(op, "expertTokenNumsOut", expertTokenNumsOut, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
+        ZB_CHECK(op, "epRecvCountsOut", epRecvCountsOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        ZB_CHECK(op, "putOffset", putOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
+        ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "expandIdxOut", expandIdxOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        /* every pick may be valid, so the packed output must hold tokens * topk rows */
+        if (quantMode == 0) {
+            ZB_CHECK(op, "expandXOut", expandXOut, x->dataType, x->dataType, T * K * H);
+        } else {
+            ZB_CHECK(op, "expandXOut", expandXOut, quantMode == 1 ? ZBAL_DATA_TYPE_INT8 : ZBAL_DATA_TYPE_FP8_E4M3,
+                     quantMode == 1 ? ZBAL_DATA_TYPE_INT8 : ZBAL_DATA_TYPE_UINT8, T * K * H);
+            ZB_CHECK(op, "dynamicScalesOut", dynamicScalesOut, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32,
+                     quantMode == 1 ? T * K : T * K * (H / 128));
+        }
+        int64_t blocks = Numel(putOffset) / E;
+        if (blocks > ZBALHIP_LAYOUT_MAX_BLOCKS) blocks = ZBALHIP_LAYOUT_MAX_BLOCKS;
+        return Launched(op, zbalhip_dispatch_low_latency(x->data, x->dataType, (const int32_t *)expertIds->data, T, H, K, E,
+                                                         (int32_t)quantMode, (int32_t)expertTokenNumsType,
+                                                         expandXOut->data, (float *)dynamicScalesOut->data,
+                                                         (int32_t *)expandIdxOut->data,
+                                                         (int64_t *)expertTokenNumsOut->data,
+                                                         (int32_t *)epRecvCountsOut->data, (int32_t *)putOffset->data,
+                                                         (int32_t)blocks, stream));
+    }
+
+    int32_t CombineLowLatency(const zbal_tensor_info_t *expandX, const zbal_tensor_info_t *expertIds,
+                              const zbal_tensor_info_t *expertIdx, const zbal_tensor_info_t *epSendCounts,
+                              const zbal_tensor_info_t *expertScales, const zbal_tensor_info_t *xOut,
+                              int64_t moeExpertNum, aclrtStream stream, int64_t) override
+    {
+        const char *op = "CombineLowlatency";
+        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        int64_t T = 0, H = 0;
+        if (!TokensShape(op, xOut, &T, &H)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(expertIds->dim == 2 && expertIds->shape[0] == T, op << " failed as expertIds must be [tokens, topk]",
+                             Z_INVALID_PARAM);
+        const int64_t K = expertIds->shape[1];
+        ZBAL_VALIDATE_RETURN(K <= 32, op << " failed as topk " << K << " exceeds 32", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN((H * 2) % 32 == 0, op << " failed as hidden " << H << " gives rows that are not a multiple of 32 bytes",
+                             Z_INVALID_PARAM);
+        if (T == 0) return Z_OK;
+        ZB_CHECK(op, "expandX", expandX, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, H);
+        ZBAL_VALIDATE_RETURN(expandX->dataType == xOut->dataType, op << " failed as source and destination types differ",
+                             Z_INVALID_PARAM);
+        ZB_CHECK(op, "xOut", xOut, expandX->dataType, expandX->dataType, T * H);
+        ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "expertIdx", expertIdx, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "epSendCounts", epSendCounts, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, moeExpertNum);
+        ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
+        return Launched(op, zbalhip_combine(expandX->data, expandX->dataType, (const int32_t *)epSendCounts->data, 1,
+                                            (const float *)expertScales->data, (const int32_t *)expertIds->data,
+                                            (const int32_t *)expertIdx->data, T, H, K, moeExpertNum, xOut->data,
+                                            stream));
+    }
+
+    int32_t FusedDeepMoe(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds,
+                         const zbal_tensor_info_t *gmm1Weight, const zbal_tensor_info_t *gmm1Scale,
+                         const zbal_tensor_info_t *gmm2Weight, const zbal_tensor_info_t *gmm2Scale,
+                         const zbal_tensor_info_t *expertScales, const zbal_tensor_info_t *expertSmoothScales,
+                         const zbal_tensor_info_t *xActiveMask, const zbal_tensor_info_t *output,
+                         const zbal_tensor_info_t *expertTokenNums, const zbal_tensor_info_t *workspace,
+                         int64_t moeExpertNum, int64_t quantMode, int64_t, int64_t gmm1HLen, aclrtStream stream,
+                         int64_t) override
+    {
+        const char *op = "FusedDeepMoe";
+        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(xActiveMask == nullptr || xActiveMask->data == nullptr,
+                             op << " failed as xActiveMask is not supported", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(quantMode >= 0 && quantMode <= 3, op << " failed as quantMode " << quantMode << " is invalid",
+                             Z_INVALID_PARAM);
+        const int mode = quantMode <= 1 ? 1 : (int)quantMode; /* 0 and 1 both mean W8A8, as in the reference kernel */
+        int64_t T = 0, H = 0;
+        if (!TokensShape(op, x, &T, &H)) return Z_INVALID_PARAM;
+        ZBAL_VALIDATE_RETURN(expertIds->dim == 2 && expertIds->shape[0] == T, op << " failed as expertIds must be [tokens, topk]",
+                             Z_INVALID_PARAM);
+        const int64_t K = expertIds->shape[1], E = moeExpertNum, N1 = gmm1HLen, I = N1 / 2;
+        ZBAL_VALIDATE_RETURN(K <= 32, op << " failed as topk " << K << " exceeds 32", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(E <= 1024, op << " failed as moeExpertNum exceeds 1024", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(N1 % 256 == 0 && H % 256 == 0,
+                             op << " failed as gmm1HLen " << N1 << " and hidden " << H << " must be multiples of 256",
+                             Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(gmm1Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_KCONTIG &&
+                                 gmm2Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_KCONTIG,
+                             op << " failed as the weights are not pre-packed (zbal_moe_weight_prepack)", Z_INVALID_PARAM);
+        const int wdt = mode == 1 ? ZBAL_DATA_TYPE_INT8 : (mode == 2 ? ZBAL_DATA_TYPE_FP8_E4M3 : ZBAL_DATA_TYPE_INT4X2);
+        const int wdt_alt = mode == 2 ? ZBAL_DATA_TYPE_UINT8 : wdt;
+        const int64_t wdiv = mode == 3 ? 2 : 1;
+        ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
+        ZB_CHECK(op, "output", output, x->dataType, x->dataType, T * H);
+        ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+        ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
+        ZB_CHECK(op, "gmm1Weight", gmm1Weight, wdt, wdt_alt, E * H * N1 / wdiv);
+        ZB_CHECK(op, "gmm2Weight", gmm2Weight, wdt, wdt_alt, E * I * H / wdiv);
+        ZB_CHECK(op, "expertTokenNums", expertTokenNums, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
+        int wscale2Dt = ZBAL_DATA_TYPE_FP32;
+        if (mode == 1) {
+            ZB_CHECK(op, "gmm1Scale", gmm1Scale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * N1);
+            ZB_CHECK(op, "gmm2Scale", gmm2Scale, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP32, E * H);
+            wscale2Dt = gmm2Scale->dataType;
+        } else if (mode == 2) {
+            ZB_CHECK(op, "gmm1Scale", gmm1Scale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * (H / 128) * (N1 / 128));
+            ZB_CHECK(op, "gmm2Scale", gmm2Scale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * (I / 128) * (H / 128));
+        } else {
+            ZB_CHECK(op, "gmm1Scale", gmm1Scale, ZBAL_DATA_TYPE_FP16, ZBAL_DATA_TYPE_FP16, E * (H / 128) * N1);
+            ZB_CHECK(op, "gmm2Scale", gmm2Scale, ZBAL_DATA_TYPE_FP16, ZBAL_DATA_TYPE_FP16, E * (I / 128) * H);
+            wscale2Dt = ZBAL_DATA_TYPE_FP16;
+        }
+        const float *smooth = nullptr;
+        if (expertSmoothScales && expertSmoothScales->data) {
+            ZBAL_VALIDATE_RETURN(mode != 2, op << " failed as smooth scales do not apply to the fp8 mode", Z_INVALID_PARAM);
+            ZB_CHECK(op, "expertSmoothScales", expertSmoothScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * H);
+            smooth = (const float *)expertSmoothScales->data;
+        }
+        FusedWorkspace ws;
+        ZBAL_VALIDATE_RETURN(PlanFusedWorkspace(T, H, K, E, N1, quantMode, &ws), op << " failed as the shapes are invalid",
+                             Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(workspace->data != nullptr && (reinterpret_cast<uintptr_t>(workspace->data) & 255u) == 0,
+                             op << " failed as the workspace is null or not 256-byte aligned", Z_INVALID_PARAM);
+        const uint64_t wsBytes = (uint64_t)Numel(workspace) * ElemSize(workspace->dataType);
+        if (wsBytes < ws.total) { /* the reference reports this case with a raw -1, host launcher :224-232 */
+            ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as the workspace holds " << wsBytes << " bytes, needs " << ws.total);
+            return Z_ERROR;
+        }
+        uint8_t *base = (uint8_t *)workspace->data;
+        const int64_t rows = T * K;
+        void *q1 = base + ws.q1;
+        float *xs = (float *)(base + ws.xs);
+        int32_t *expandIdx = (int32_t *)(base + ws.expand_idx);
+        int32_t *rowOff = (int32_t *)(base + ws.row_off);
+        int32_t *scratch = (int32_t *)(base + ws.layout_scratch);
+        void *q2 = base + ws.q2;
+        float *scale2 = (float *)(base + ws.scale2);
+        float *sgl = mode == 2 ? nullptr : (float *)(base + ws.sgl);
+        void *y = base + ws.y;
+        if (T == 0) { /* nothing routed: counts are zero */
+            return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, 0,
+                                                            H, K, E, mode == 2 ? 2 : 1, q1, xs, expandIdx,
+                                                            (int64_t *)expertTokenNums->data, rowOff, scratch,
+                                                            ZBALHIP_LAYOUT_MAX_BLOCKS, stream));
+        }
+        int32_t rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, T, H, K, E,
+                                                 mode == 2 ? 2 : 1, q1, xs, expandIdx, (int64_t *)expertTokenNums->data,
+                                                 rowOff, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
+        if (rc != 0) return Launched(op, rc);
+        rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1, mode, q2, scale2,
+                                       sgl, stream);
+        if (rc != 0) return Launched(op, rc);
+        rc = zbalhip_gmm2_dequant(q2, scale2, gmm2Weight->data, gmm2Scale->data, wscale2Dt, rowOff, E, rows, I, H, mode,
+                                  x->dataType, y, stream);
+        if (rc != 0) return Launched(op, rc);
+        return Launched(op, zbalhip_combine(y, x->dataType, rowOff, 0, (const float *)expertScales->data,
+                                            (const int32_t *)expertIds->data, expandIdx, T, H, K, E, output->data,
+                                            stream));
+    }
+
+    int32_t TopkRoute(const zbal_tensor_info_t *logits, int64_t topkNum, const zbal_tensor_info_t *topkIndex,
+                      const zbal_tensor_info_t *topkWeight, aclrtStream stream, int64_t) override
+    {
+        const char *op = "TopkRoute";
+        ZBAL_VALIDATE_RETURN(logits->dim == 2, op << " failed as logits must be [tokens, experts]", Z_INVALID_PARAM);
+        const int64_t T = logits->shape[0], E = logits->shape[1];
+        ZBAL_VALIDATE_RETURN(E > 0 && E <= 1024 && topkNum <= 32 && topkNum <= E,
+                             op << " failed as experts " << E << " / topk " << topkNum << " are out of range", Z_INVALID_PARAM);
+        if (T == 0) return Z_OK;
+        ZB_CHECK(op, "logits", logits, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * E);
+        ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, T * topkNum);
+        ZB_CHECK(op, "topkWeight", topkWeight, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * topkNum);
+        return Launched(op, zbalhip_topk_route((const float *)logits->data, T, E, topkNum, (int64_t *)topkIndex->data,
+                                               (float *)topkWeight->data, stream));
+    }
+
+    int32_t WeightPrepack(const zbal_tensor_info_t *src, const zbal_tensor_info_t *dst, aclrtStream stream, int64_t) override
+    {
+        const char *op = "WeightPrepack";
+        ZBAL_VALIDATE_RETURN(src->dim == 3, op << " failed as src must be [experts, K, N]", Z_INVALID_PARAM);
+        const int64_t E = src->shape[0], K = src->shape[1], N = src->shape[2];
+        const bool int4 = dst->dataType == ZBAL_DATA_TYPE_INT4X2;
+        ZBAL_VALIDATE_RETURN(ElemSize(src->dataType) == 1, op << " failed as src must hold one byte per element", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(!int4 || src->dataType == ZBAL_DATA_TYPE_INT8, op << " failed as int4 packing needs an int8 source",
+                             Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(src->data && dst->data && src->data != dst->data, op << " failed as src/dst are null or alias",
+                             Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(Numel(dst) * (int4 ? 2 : 1) >= E * K * N, op << " failed as dst is too small", Z_INVALID_PARAM);
+        return Launched(op, zbalhip_weight_prepack(src->data, E, K, N, int4 ? 1 : 0, dst->data, stream));
+    }
+};
+
+} // namespace
+
+CommunicatorPtr MakeGpuCommunicator(const GroupInfo &info) { return std::make_shared<GpuCommunicator>(info); }
+
+static uint64_t Align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
+
+bool PlanFusedWorkspace(int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int64_t n1, int64_t quantMode,
+                        FusedWorkspace *ws)
+{
+    if (tokens < 0 || hidden <= 0 || topk <= 0 || experts <= 0 || n1 <= 0 || quantMode < 0 || quantMode > 3) return false;
+    if (hidden % 128 != 0 || n1 % 256 != 0) return false;
+    const uint64_t rows = (uint64_t)(tokens * topk > 0 ? tokens * topk : 1);
+    const uint64_t H = hidden, I = n1 / 2, E = experts;
+    const bool fp8 = quantMode == 2;
+    uint64_t off = 0;
+    auto take = [&](uint64_t bytes) { uint64_t o = off; off = Align256(off + bytes); return o; };
+    ws->q1 = take(rows * H);
+    ws->xs = take(rows * (fp8 ? H / 128 : 1) * 4);
+    ws->expand_idx = take(rows * 4);
+    ws->counts = take(E * 8);
+    ws->row_off = take((E + 1) * 4);
+    ws->layout_scratch = take((uint64_t)ZBALHIP_LAYOUT_MAX_BLOCKS * E * 4);
+    ws->q2 = take(rows * I);
+    ws->scale2 = take(rows * (fp8 ? (I + 127) / 128 : 1) * 4);
+    ws->sgl = fp8 ? off : take(rows * (I + 1) * 4);
+    ws->y = take(rows * H * 2);
+    ws->total = off;
+    return true;
+}
+
+} // namespace zbal

@@ -1,0 +1,103 @@
+/*
+ * Weighted combine (gather-reduce): out[t,:] = round(sum_k w[t,k] * y[row(t,k),:]).
+ *
+ * One workgroup per output token. Each lane owns 16-byte chunks (8 elements)
+ * of the row; for a chunk it issues the loads of up to eight picks back to
+ * back so that eight 16-byte requests per lane are in flight, then folds
+ * them into fp32 accumulators in pick order with a separately rounded
+ * multiply and add, and stores one rounded 16-byte chunk. HBM traffic is
+ * K row reads plus one row write per token.
+ */
+#include "zbal_device.h"
+#include "zbal_hip_kernels.h"
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kMaxTopk = 32;
+constexpr int kGroup = 8;
+
+template <int DT>
+__global__ void __launch_bounds__(kThreads)
+combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base, int base_inclusive,
+               const float *__restrict__ w, const int32_t *__restrict__ topk_idx,
+               const int32_t *__restrict__ rank_in_expert, int hidden, int topk, int experts,
+               uint16_t *__restrict__ out)
+{
+    __shared__ int64_t s_row[kMaxTopk];
+    __shared__ float s_w[kMaxTopk];
+    __shared__ int s_n;
+    const int t = blockIdx.x;
+    if (threadIdx.x == 0) {
+        /* compact the valid picks, keeping their order */
+        int n = 0;
+        for (int k = 0; k < topk; ++k) {
+            const int e = topk_idx[(int64_t)t * topk + k];
+            if (e < 0 || e >= experts) continue;
+            const int32_t b = base_inclusive ? (e == 0 ? 0 : base[e - 1]) : base[e];
+            s_row[n] = (int64_t)b + rank_in_expert[(int64_t)t * topk + k];
+            s_w[n] = w[(int64_t)t * topk + k];
+            ++n;
+        }
+        s_n = n;
+    }
+    __syncthreads();
+    const int n = s_n;
+    const int nchunk = hidden / 8;
+    for (int c = threadIdx.x; c < nchunk; c += blockDim.x) {
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+        for (int k0 = 0; k0 < n; k0 += kGroup) {
+            u32x4 v[kGroup];
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u)
+                if (k0 + u < n)
+                    v[u] = __builtin_nontemporal_load(
+                        reinterpret_cast<const u32x4 *>(y + s_row[k0 + u] * hidden + (int64_t)c * 8));
+#pragma unroll
+            for (int u = 0; u < kGroup; ++u) {
+                if (k0 + u < n) {
+                    const float wk = s_w[k0 + u];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float lo = zb_half_to_f32<DT>(v[u][i] & 0xffffu) * wk;
+                        const float hi = zb_half_to_f32<DT>(v[u][i] >> 16) * wk;
+                        acc[2 * i] = acc[2 * i] + lo;
+                        acc[2 * i + 1] = acc[2 * i + 1] + hi;
+                    }
+                }
+            }
+        }
+        u32x4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = zb_f32_to_half<DT>(acc[2 * i]) | (zb_f32_to_half<DT>(acc[2 * i + 1]) << 16);
+        __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(out + (int64_t)t * hidden + (int64_t)c * 8));
+    }
+}
+
+} // namespace
+
+extern "C" int32_t zbalhip_combine(const void *y, int32_t dtype, const int32_t *base, int32_t base_is_inclusive,
+                                   const float *w, const int32_t *topk_idx, const int32_t *send_token_idx,
+                                   int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, void *out,
+                                   void *stream)
+{
+    if (!y || !base || !w || !topk_idx || !send_token_idx || !out) return ZBALHIP_INVALID;
+    if (dtype != ZDT_BF16 && dtype != ZDT_FP16) return ZBALHIP_INVALID;
+    if (tokens < 0 || hidden <= 0 || hidden % 8 != 0 || topk <= 0 || topk > kMaxTopk || experts <= 0)
+        return ZBALHIP_INVALID;
+    if (tokens == 0) return ZBALHIP_OK;
+    int threads = (int)((hidden / 8 + 63) / 64 * 64);
+    if (threads > kThreads) threads = kThreads;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == ZDT_BF16)
+        combine_kernel<ZDT_BF16><<<(unsigned)tokens, threads, 0, st>>>((const uint16_t *)y, base, base_is_inclusive, w,
+                                                                     topk_idx, send_token_idx, (int)hidden, (int)topk,
+                                                                     (int)experts, (uint16_t *)out);
+    else
+        combine_kernel<ZDT_FP16><<<(unsigned)tokens, threads, 0, st>>>((const uint16_t *)y, base, base_is_inclusive, w,
+                                                                     topk_idx, send_token_idx, (int)hidden, (int)topk,
+                                                                     (int)experts, (uint16_t *)out);
+    return zbalhip_check_launch();
+}

@@ -1,0 +1,561 @@
+/*
+ * Grouped (per-expert, ragged-M) quantised GEMM with fused epilogues for gfx950.
+ *
+ * Operands: activations A [rows, K] one byte per element (int8 or e4m3),
+ * expert-major rows delimited by row_off[E+1]; weights W pre-packed
+ * [E, N, K] with K contiguous (int4: [E, N, K/2]). Both operands are
+ * K-contiguous, so either can feed either MFMA input; the kernel feeds the
+ * WEIGHT fragment as the matrix-A input and the ACTIVATION fragment as the
+ * matrix-B input, i.e. it computes C^T. With the 16x16 MFMA output layout
+ * (lane l holds output column l%16, rows 4*(l/16)+i) every lane then owns ONE
+ * token row and FOUR consecutive output channels per instruction: per-token
+ * scales are one value per lane, per-channel scales a 16-byte vector, gate/up
+ * pairs of the SwiGLU sit in the same lane, and results leave as 4-element
+ * vectors.
+ *
+ * Workgroup tile: 128 token rows x 256 output channels x 128 K-bytes, four
+ * waves in a 2x2 grid, each wave 64 rows x 128 channels = 4x8 MFMA tiles
+ * (128 accumulator registers). For GMM1 the 256 channels are 128 gate
+ * columns j and the matching 128 up columns I+j, so the SwiGLU product and,
+ * in the fp8 mode, the complete 1x128 requantisation happen in registers.
+ * A and W tiles are staged in LDS (rows padded by 16 bytes so that the
+ * 16-byte fragment reads of 16 consecutive rows fall in distinct banks);
+ * the next K-slab is fetched from HBM into registers while the current one
+ * is multiplied (two workgroups per CU hide the barriers).
+ *
+ * Tile schedule: workgroup ids are dealt round-robin to the 8 XCDs by the
+ * hardware, so id -> (id % 8) * chunk + id / 8 gives every XCD a contiguous
+ * run of logical tiles; logical tiles walk an expert in groups of
+ * (all its row tiles) x (8 channel tiles), row tile fastest, so the ~64
+ * workgroups resident on an XCD share both their A and their W slabs in
+ * that XCD's L2.
+ */
+#include "zbal_device.h"
+#include "zbal_hip_kernels.h"
+
+namespace {
+
+constexpr int BM = 128;          /* token rows per workgroup tile */
+constexpr int BN = 256;          /* output channels per workgroup tile */
+constexpr int BKB = 128;         /* K bytes per slab (128 int8/e4m3 elements) */
+constexpr int LDS_STRIDE = BKB + 16;
+constexpr int GROUP_N = 8;       /* channel tiles per schedule group */
+constexpr int kThreads = 256;
+
+enum { MODE_W8A8 = 1, MODE_FP8 = 2, MODE_W4A8 = 3 };
+
+struct GemmParams {
+    const uint8_t *a;        /* [rows, K] */
+    const float *a_scale;    /* [rows] or [rows, K/128] */
+    const uint8_t *w;        /* [E, N, K] or [E, N, K/2] */
+    const void *wscale;
+    const int32_t *row_off;  /* [E+1] */
+    int experts;
+    int max_rows;            /* rows the A / output buffers hold */
+    int K;
+    int N;                   /* weight rows per expert (N1 for GMM1) */
+    int wscale_is_bf16;
+    void *out;               /* GMM1: q2 bytes; GMM2: y */
+    float *out_scale;        /* GMM1: scale2 (fp8 mode) */
+    float *sgl_ws;           /* GMM1 int8 modes: fp32 SwiGLU values [rows, N/2] */
+    uint32_t *rowmax;        /* GMM1 int8 modes: per-row absmax bits */
+};
+
+struct TileCoord {
+    int expert, m_tile, n_tile;
+};
+
+/* wave-uniform search of the logical tile this workgroup owns; false = nothing to do */
+__device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ row_off, int experts, int n_tiles,
+                                            TileCoord &tc)
+{
+    const int lane = threadIdx.x & 63;
+    int total = 0;
+    for (int base = 0; base < experts; base += 64) {
+        const int e = base + lane;
+        int t = 0;
+        if (e < experts) t = ((row_off[e + 1] - row_off[e] + BM - 1) / BM) * n_tiles;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
+        total += t;
+    }
+    const int chunk = (total + 7) / 8;
+    const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
+    if (slot >= chunk) return false;
+    const int lid = xcd * chunk + slot;
+    if (lid >= total) return false;
+
+    int run = 0, expert = -1, start = 0, mt_e = 0;
+    for (int base = 0; base < experts; base += 64) {
+        const int e = base + lane;
+        int mt = 0;
+        if (e < experts) mt = (row_off[e + 1] - row_off[e] + BM - 1) / BM;
+        const int t = mt * n_tiles;
+        int incl = t;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int o = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += o;
+        }
+        const int excl = run + incl - t;
+        const bool hit = t > 0 && lid >= excl && lid < excl + t;
+        const uint64_t bal = __ballot(hit);
+        if (bal) {
+            const int src = __ffsll((long long)bal) - 1;
+            expert = base + src;
+            start = __shfl(excl, src, 64);
+            mt_e = __shfl(mt, src, 64);
+            break;
+        }
+        run += __shfl(incl, 63, 64);
+    }
+    if (expert < 0) return false;
+    const int l = lid - start;
+    const int per_group = mt_e * GROUP_N;
+    const int ng = l / per_group;
+    const int r = l - ng * per_group;
+    tc.expert = expert;
+    tc.m_tile = r % mt_e;
+    tc.n_tile = ng * GROUP_N + r / mt_e;
+    return true;
+}
+
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ f32x4 mfma_fp8_16x16x128(const i32x8 &wfrag, const i32x8 &afrag)
+{
+    const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
+    /* cbsz = blgp = 0 selects e4m3 for both inputs; scale exponents 0 leave the product unscaled */
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(wfrag, afrag, zero, 0, 0, 0, 0, 0, 0);
+}
+
+/* four consecutive bytes -> one dword store helpers */
+__device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d)
+{
+    return zb_cvt_pk_e4m3(a, b) | (zb_cvt_pk_e4m3(c, d) << 16);
+}
+
+template <int MODE, bool GMM1, int OUT_DT>
+__global__ void __launch_bounds__(kThreads, 2)
+grouped_gemm_kernel(GemmParams p)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t lds_a[BM * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) uint8_t lds_w[BN * LDS_STRIDE];
+    __shared__ __attribute__((aligned(16))) float lds_sa[BM];          /* fp8: activation scales of the slab */
+    __shared__ __attribute__((aligned(16))) float lds_gs[BN];          /* W4A8: group scales of the slab / 16 */
+    __shared__ float lds_rowmax[2][BM];
+
+    const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
+    TileCoord tc;
+    if (!locate_tile(p.row_off, p.experts, n_tiles, tc)) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int row_begin = p.row_off[tc.expert] + tc.m_tile * BM;
+    const int row_end = p.row_off[tc.expert + 1];
+    const int K = p.K;
+    const int KB = K / 128;
+    const int I = p.N / 2;
+
+    /* ---- global -> register staging ------------------------------------------------ */
+    constexpr int A_LOADS = BM * (BKB / 16) / kThreads;                         /* 4 */
+    constexpr int W_BYTES_ROW = (MODE == MODE_W4A8) ? BKB / 2 : BKB;            /* bytes of one W row per slab */
+    constexpr int W_LOADS = BN * (W_BYTES_ROW / 16) / kThreads;                 /* 8 or 4 */
+    const uint8_t *a_ptr[A_LOADS];
+    const uint8_t *w_ptr[W_LOADS];
+    int a_lds[A_LOADS], w_lds[W_LOADS];
+#pragma unroll
+    for (int i = 0; i < A_LOADS; ++i) {
+        const int q = tid + i * kThreads, r = q >> 3, c = q & 7;
+        int gr = row_begin + r;
+        if (gr > p.max_rows - 1) gr = p.max_rows - 1;
+        a_ptr[i] = p.a + (int64_t)gr * K + c * 16;
+        a_lds[i] = r * LDS_STRIDE + c * 16;
+    }
+    const int64_t w_row_bytes = (MODE == MODE_W4A8) ? K / 2 : K;
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+        constexpr int CPR = W_BYTES_ROW / 16; /* chunks per row */
+        const int q = tid + i * kThreads, r = q / CPR, c = q % CPR;
+        int wrow;
+        if (GMM1) wrow = (r < 128) ? tc.n_tile * 128 + r : I + tc.n_tile * 128 + (r - 128);
+        else wrow = tc.n_tile * BN + r;
+        w_ptr[i] = p.w + ((int64_t)tc.expert * p.N + wrow) * w_row_bytes + c * 16;
+        w_lds[i] = r * LDS_STRIDE + c * ((MODE == MODE_W4A8) ? 32 : 16);
+    }
+    /* per-slab scale staging */
+    const float *sa_ptr = nullptr;
+    if (MODE == MODE_FP8 && tid < BM) {
+        int gr = row_begin + tid;
+        if (gr > p.max_rows - 1) gr = p.max_rows - 1;
+        sa_ptr = p.a_scale + (int64_t)gr * KB;
+    }
+    const uint16_t *gs_ptr = nullptr;
+    if (MODE == MODE_W4A8) {
+        int wrow;
+        if (GMM1) wrow = (tid < 128) ? tc.n_tile * 128 + tid : I + tc.n_tile * 128 + (tid - 128);
+        else wrow = tc.n_tile * BN + tid;
+        gs_ptr = (const uint16_t *)p.wscale + (int64_t)tc.expert * KB * p.N + wrow;
+    }
+    /* fp8 weight block scales: two per slab for this tile */
+    const float *sw_ptr0 = nullptr, *sw_ptr1 = nullptr;
+    if (MODE == MODE_FP8) {
+        const int NB = p.N / 128;
+        const float *base = (const float *)p.wscale + (int64_t)tc.expert * KB * NB;
+        if (GMM1) { sw_ptr0 = base + tc.n_tile; sw_ptr1 = base + I / 128 + tc.n_tile; }
+        else { sw_ptr0 = base + tc.n_tile * 2; sw_ptr1 = sw_ptr0 + 1; }
+    }
+
+    u32x4 a_reg[A_LOADS], w_reg[W_LOADS];
+    float sa_reg = 0.0f, gs_reg = 0.0f;
+    auto fetch = [&](int kb) {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) a_reg[i] = *reinterpret_cast<const u32x4 *>(a_ptr[i] + (int64_t)kb * BKB);
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i)
+            w_reg[i] = *reinterpret_cast<const u32x4 *>(w_ptr[i] + (int64_t)kb * W_BYTES_ROW);
+        if (MODE == MODE_FP8 && tid < BM) sa_reg = sa_ptr[kb];
+        if (MODE == MODE_W4A8) gs_reg = zb_fp16_to_f32(gs_ptr[(int64_t)kb * p.N]) * 0.0625f;
+    };
+    auto stash = [&]() {
+#pragma unroll
+        for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<u32x4 *>(lds_a + a_lds[i]) = a_reg[i];
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i) {
+            if constexpr (MODE == MODE_W4A8) {
+                /* byte b of each dword holds k[b] (low nibble) and k[b+4] (high nibble); <<4 keeps the sign
+                   and multiplies by 16, undone in the group scale */
+                u32x4 lo, hi;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    lo[j] = (w_reg[i][j] << 4) & 0xf0f0f0f0u;
+                    hi[j] = w_reg[i][j] & 0xf0f0f0f0u;
+                }
+                u32x4 o0 = {lo[0], hi[0], lo[1], hi[1]};
+                u32x4 o1 = {lo[2], hi[2], lo[3], hi[3]};
+                *reinterpret_cast<u32x4 *>(lds_w + w_lds[i]) = o0;
+                *reinterpret_cast<u32x4 *>(lds_w + w_lds[i] + 16) = o1;
+            } else {
+                *reinterpret_cast<u32x4 *>(lds_w + w_lds[i]) = w_reg[i];
+            }
+        }
+        if (MODE == MODE_FP8 && tid < BM) lds_sa[tid] = sa_reg;
+        if (MODE == MODE_W4A8) lds_gs[tid] = gs_reg;
+    };
+
+    /* ---- accumulators ------------------------------------------------------------------ */
+    f32x4 accf[4][8];
+    i32x4 acci[4][8];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) {
+            accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            acci[mt][nt] = i32x4{0, 0, 0, 0};
+        }
+
+    /* fragment addresses: lane reads row (lane%16) of a 16-row sub-tile, K bytes [32*(lane/16), +32) */
+    const int frag_row = lane & 15, frag_k = (lane >> 4) * 32;
+    int a_frag_off[4], w_frag_off[8];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) a_frag_off[mt] = (wm * 64 + mt * 16 + frag_row) * LDS_STRIDE + frag_k;
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) {
+        int r;
+        if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
+        else r = wn * 128 + nt * 16;
+        w_frag_off[nt] = (r + frag_row) * LDS_STRIDE + frag_k;
+    }
+
+    fetch(0);
+    for (int kb = 0; kb < KB; ++kb) {
+        __syncthreads();
+        stash();
+        __syncthreads();
+        if (kb + 1 < KB) fetch(kb + 1);
+
+        if constexpr (MODE == MODE_FP8) {
+            const float sw0 = sw_ptr0[(int64_t)kb * (p.N / 128)], sw1 = sw_ptr1[(int64_t)kb * (p.N / 128)];
+            i32x8 af[4];
+            float s0[4], s1[4];
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds_a + a_frag_off[mt]);
+                const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds_a + a_frag_off[mt] + 16);
+                af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                const float sa = lds_sa[wm * 64 + mt * 16 + frag_row];
+                s0[mt] = sa * sw0;
+                s1[mt] = sa * sw1;
+            }
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) {
+                const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds_w + w_frag_off[nt]);
+                const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds_w + w_frag_off[nt] + 16);
+                const i32x8 wf = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                const bool second = GMM1 ? (nt >= 4) : (wn == 1);
+#pragma unroll
+                for (int mt = 0; mt < 4; ++mt) {
+                    const f32x4 part = mfma_fp8_16x16x128(wf, af[mt]);
+                    const float s = second ? s1[mt] : s0[mt];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], s, accf[mt][nt][i]);
+                }
+            }
+        } else {
+            /* int8 operands: two 64-deep MFMA steps per slab; lane's K bytes are [32*(lane/16) + 16*h, +16) */
+            i32x4 af[4][2];
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(lds_a + a_frag_off[mt] + 16 * h);
+                    af[mt][h] = i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
+                }
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) {
+                i32x4 wf[2];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const u32x4 v = *reinterpret_cast<const u32x4 *>(lds_w + w_frag_off[nt] + 16 * h);
+                    wf[h] = i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
+                }
+                if constexpr (MODE == MODE_W8A8) {
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) {
+                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0], af[mt][0], acci[mt][nt], 0, 0, 0);
+                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[1], af[mt][1], acci[mt][nt], 0, 0, 0);
+                    }
+                } else {
+                    int r;
+                    if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
+                    else r = wn * 128 + nt * 16;
+                    const f32x4 gs = *reinterpret_cast<const f32x4 *>(&lds_gs[r + (lane >> 4) * 4]);
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) {
+                        i32x4 part = i32x4{0, 0, 0, 0};
+                        part = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0], af[mt][0], part, 0, 0, 0);
+                        part = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[1], af[mt][1], part, 0, 0, 0);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i)
+                            accf[mt][nt][i] = __builtin_fmaf((float)part[i], gs[i], accf[mt][nt][i]);
+                    }
+                }
+            }
+        }
+    }
+
+    /* ---- epilogue ------------------------------------------------------------------------- */
+    /* lane owns token row m = row_begin + wm*64 + mt*16 + lane%16 and channels 4*(lane/16)+i of each 16-wide sub-tile */
+    const int sub_n = (lane >> 4) * 4;
+    if constexpr (!GMM1) {
+        uint16_t *y = (uint16_t *)p.out;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
+            if (row >= row_end) continue;
+            float xs = 1.0f;
+            if (MODE != MODE_FP8) xs = p.a_scale[row];
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) {
+                const int n = tc.n_tile * BN + wn * 128 + nt * 16 + sub_n;
+                float d[4];
+                if constexpr (MODE == MODE_W8A8) {
+                    float ws[4];
+                    if (p.wscale_is_bf16) {
+                        const u32x2 v = *reinterpret_cast<const u32x2 *>((const uint16_t *)p.wscale + (int64_t)tc.expert * p.N + n);
+                        ws[0] = zb_bf16_to_f32(v[0] & 0xffffu); ws[1] = zb_bf16_to_f32(v[0] >> 16);
+                        ws[2] = zb_bf16_to_f32(v[1] & 0xffffu); ws[3] = zb_bf16_to_f32(v[1] >> 16);
+                    } else {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>((const float *)p.wscale + (int64_t)tc.expert * p.N + n);
+                        ws[0] = v[0]; ws[1] = v[1]; ws[2] = v[2]; ws[3] = v[3];
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) d[i] = ((float)acci[mt][nt][i] * ws[i]) * xs;
+                } else if constexpr (MODE == MODE_FP8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i] * xs;
+                }
+                u32x2 o;
+                o[0] = zb_f32_to_half<OUT_DT>(d[0]) | (zb_f32_to_half<OUT_DT>(d[1]) << 16);
+                o[1] = zb_f32_to_half<OUT_DT>(d[2]) | (zb_f32_to_half<OUT_DT>(d[3]) << 16);
+                *reinterpret_cast<u32x2 *>(y + (int64_t)row * p.N + n) = o;
+            }
+        }
+    } else {
+        /* SwiGLU on gate sub-tile nt and up sub-tile nt+4: columns j = n_tile*128 + wn*64 + nt*16 + sub_n + i */
+        float sg[4][4][4];
+        float rmax[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
+            int lrow = row;
+            if (lrow > p.max_rows - 1) lrow = p.max_rows - 1;
+            float xs = 1.0f;
+            if (MODE != MODE_FP8) xs = p.a_scale[lrow];
+            rmax[mt] = 0.0f;
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                float g[4], u[4];
+                if constexpr (MODE == MODE_W8A8) {
+                    const float *wsb = (const float *)p.wscale + (int64_t)tc.expert * p.N;
+                    const f32x4 wg = *reinterpret_cast<const f32x4 *>(wsb + j);
+                    const f32x4 wu = *reinterpret_cast<const f32x4 *>(wsb + I + j);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        g[i] = ((float)acci[mt][nt][i] * wg[i]) * xs;
+                        u[i] = ((float)acci[mt][nt + 4][i] * wu[i]) * xs;
+                    }
+                } else if constexpr (MODE == MODE_FP8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { g[i] = accf[mt][nt][i]; u[i] = accf[mt][nt + 4][i]; }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { g[i] = accf[mt][nt][i] * xs; u[i] = accf[mt][nt + 4][i] * xs; }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float left = g[i] / (1.0f + zb_expf(-g[i]));
+                    const float s = left * u[i];
+                    sg[mt][nt][i] = s;
+                    rmax[mt] = fmaxf(rmax[mt], fabsf(s));
+                }
+            }
+            /* the four lane groups (lane/16) hold different columns of the same row */
+            rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 16, 64));
+            rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 32, 64));
+            if (lane < 16) lds_rowmax[wn][wm * 64 + mt * 16 + lane] = rmax[mt];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const int lr = wm * 64 + mt * 16 + frag_row;
+            const int row = row_begin + lr;
+            const float amax_tile = fmaxf(lds_rowmax[0][lr], lds_rowmax[1][lr]);
+            if (row >= row_end) continue;
+            if constexpr (MODE == MODE_FP8) {
+                const float amax = fmaxf(amax_tile, 1e-4f);
+                const float mult = 448.0f / amax;
+                uint8_t *q2 = (uint8_t *)p.out;
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                    const uint32_t v = pack4_e4m3(sg[mt][nt][0] * mult, sg[mt][nt][1] * mult, sg[mt][nt][2] * mult,
+                                                  sg[mt][nt][3] * mult);
+                    *reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I + j) = v;
+                }
+                if (wn == 0 && lane < 16) p.out_scale[(int64_t)row * (I / 128) + tc.n_tile] = amax * (1.0f / 448.0f);
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                    const f32x4 v = f32x4{sg[mt][nt][0], sg[mt][nt][1], sg[mt][nt][2], sg[mt][nt][3]};
+                    *reinterpret_cast<f32x4 *>(p.sgl_ws + (int64_t)row * I + j) = v;
+                }
+                if (wn == 0 && lane < 16) atomicMax(&p.rowmax[row], __float_as_uint(amax_tile));
+            }
+        }
+    }
+}
+
+/* second pass of the int8 GMM1 epilogue: whole-row requantisation from the fp32 SwiGLU values */
+__global__ void __launch_bounds__(256)
+requant_rows_kernel(const float *__restrict__ sgl, const uint32_t *__restrict__ rowmax, const int32_t *__restrict__ row_off,
+                    int experts, int I, int8_t *__restrict__ q2, float *__restrict__ scale2)
+{
+    const int total = row_off[experts];
+    for (int row = blockIdx.x; row < total; row += gridDim.x) {
+        const float mx = __uint_as_float(rowmax[row]);
+        const float inv = mx == 0.0f ? 0.0f : 1.0f / mx;
+        if (threadIdx.x == 0) scale2[row] = mx * (1.0f / 127.0f);
+        for (int c = threadIdx.x; c < I / 4; c += blockDim.x) {
+            const f32x4 v = *reinterpret_cast<const f32x4 *>(sgl + (int64_t)row * I + c * 4);
+            uint32_t w = 0;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) w |= ((uint32_t)zb_rint_i8((v[i] * 127.0f) * inv) & 0xffu) << (8 * i);
+            *reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I + c * 4) = w;
+        }
+    }
+}
+
+__global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
+inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles)
+{
+    int64_t m_tiles = (max_rows + BM - 1) / BM + experts;   /* each expert adds at most one partial tile */
+    int64_t g = m_tiles * n_tiles;
+    return (unsigned)((g + 7) / 8 * 8);
+}
+
+} // namespace
+
+extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale, const void *w1, const void *w1scale,
+                                             const int32_t *row_off, int64_t experts, int64_t max_rows, int64_t k,
+                                             int64_t n1, int32_t mode, void *q2, float *scale2, float *sgl_ws,
+                                             void *stream)
+{
+    if (!a || !a_scale || !w1 || !w1scale || !row_off || !q2 || !scale2) return ZBALHIP_INVALID;
+    if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
+    if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || n1 <= 0 || n1 % 256 != 0)
+        return ZBALHIP_INVALID;
+    if (max_rows == 0) return ZBALHIP_OK;
+    hipStream_t st = (hipStream_t)stream;
+    GemmParams p = {};
+    p.a = (const uint8_t *)a; p.a_scale = a_scale; p.w = (const uint8_t *)w1; p.wscale = w1scale; p.row_off = row_off;
+    p.experts = (int)experts; p.max_rows = (int)max_rows; p.K = (int)k; p.N = (int)n1;
+    p.out = q2; p.out_scale = scale2; p.sgl_ws = sgl_ws;
+    const int n_tiles = (int)(n1 / 2 / 128);
+    const unsigned grid = grid_for(max_rows, experts, n_tiles);
+    if (mode == MODE_FP8) {
+        grouped_gemm_kernel<MODE_FP8, true, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
+        return zbalhip_check_launch();
+    }
+    if (!sgl_ws) return ZBALHIP_INVALID;
+    /* the row maxima live behind the SwiGLU values in the same scratch allocation */
+    p.rowmax = (uint32_t *)(sgl_ws + max_rows * (n1 / 2));
+    fill_u32_kernel<<<(unsigned)((max_rows + 255) / 256), 256, 0, st>>>(p.rowmax, max_rows, 0u);
+    if (mode == MODE_W8A8) grouped_gemm_kernel<MODE_W8A8, true, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
+    else grouped_gemm_kernel<MODE_W4A8, true, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
+    int64_t rb = max_rows < 4096 ? max_rows : 4096;
+    requant_rows_kernel<<<(unsigned)rb, 256, 0, st>>>(sgl_ws, p.rowmax, row_off, (int)experts, (int)(n1 / 2),
+                                                    (int8_t *)q2, scale2);
+    return zbalhip_check_launch();
+}
+
+extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, const void *w2, const void *wscale,
+                                        int32_t wscale_dtype, const int32_t *row_off, int64_t experts,
+                                        int64_t max_rows, int64_t k, int64_t n, int32_t mode, int32_t out_dtype,
+                                        void *y, void *stream)
+{
+    if (!a || !a_scale || !w2 || !wscale || !row_off || !y) return ZBALHIP_INVALID;
+    if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
+    if (out_dtype != ZDT_BF16 && out_dtype != ZDT_FP16) return ZBALHIP_INVALID;
+    if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || n <= 0 || n % BN != 0)
+        return ZBALHIP_INVALID;
+    if (mode == MODE_W8A8 && wscale_dtype != ZDT_FP32 && wscale_dtype != ZDT_BF16) return ZBALHIP_INVALID;
+    if (max_rows == 0) return ZBALHIP_OK;
+    hipStream_t st = (hipStream_t)stream;
+    GemmParams p = {};
+    p.a = (const uint8_t *)a; p.a_scale = a_scale; p.w = (const uint8_t *)w2; p.wscale = wscale; p.row_off = row_off;
+    p.experts = (int)experts; p.max_rows = (int)max_rows; p.K = (int)k; p.N = (int)n;
+    p.wscale_is_bf16 = (wscale_dtype == ZDT_BF16);
+    p.out = y;
+    const unsigned grid = grid_for(max_rows, experts, (int)(n / BN));
+    const bool bf = out_dtype == ZDT_BF16;
+#define ZB_GO(M)                                                                            \
+    do {                                                                                    \
+        if (bf) grouped_gemm_kernel<M, false, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);      \
+        else grouped_gemm_kernel<M, false, ZDT_FP16><<<grid, kThreads, 0, st>>>(p);         \
+    } while (0)
+    if (mode == MODE_W8A8) ZB_GO(MODE_W8A8);
+    else if (mode == MODE_FP8) ZB_GO(MODE_FP8);
+    else ZB_GO(MODE_W4A8);
+#undef ZB_GO
+    return zbalhip_check_launch();
+}

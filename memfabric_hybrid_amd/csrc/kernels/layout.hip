@@ -1,0 +1,339 @@
+/*
+ * Routing and layout kernels: softmax top-k router, per-expert histogram with
+ * stable per-pick ranks, and the count scans that turn the histogram into row
+ * offsets.
+ *
+ * The stable rank of a pick (its position among earlier picks of the same
+ * expert, in flat (t,k) order) is computed without atomics on the result:
+ * blocks own contiguous token ranges, a first pass leaves one histogram per
+ * block in `scratch`, and the second pass starts each block from the sum of
+ * the histograms of the blocks before it; inside a block, picks are ranked 64
+ * at a time with wave ballots (lanes holding the same expert find each other
+ * by intersecting one ballot per index bit) and the four waves of a block
+ * commit their running counts in wave order.
+ */
+#include "zbal_device.h"
+#include "zbal_hip_kernels.h"
+
+#define ZB_MAX_EXPERTS 1024
+#define ZB_LAYOUT_THREADS 256
+
+namespace {
+
+struct LayoutPlan {
+    int nblk;
+    int tokens_per_block;
+};
+
+inline LayoutPlan plan_layout(int64_t tokens, int64_t topk, int max_blocks)
+{
+    LayoutPlan p;
+    int64_t want = (tokens * topk + 1023) / 1024;
+    if (want < 1) want = 1;
+    if (want > max_blocks) want = max_blocks;
+    int64_t tpb = (tokens + want - 1) / want;
+    if (tpb < 1) tpb = 1;
+    p.tokens_per_block = (int)tpb;
+    p.nblk = (int)((tokens + tpb - 1) / tpb);
+    if (p.nblk < 1) p.nblk = 1;
+    return p;
+}
+
+template <typename IdxT>
+__global__ void __launch_bounds__(ZB_LAYOUT_THREADS)
+layout_hist_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int experts, int ranks, int tpb,
+                   int32_t *__restrict__ scratch, int32_t *__restrict__ tokens_per_rank)
+{
+    __shared__ int32_t hist[ZB_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) hist[e] = 0;
+    if (blockIdx.x == 0 && tokens_per_rank)
+        for (int r = threadIdx.x; r < ranks; r += blockDim.x) tokens_per_rank[r] = 0;
+    __syncthreads();
+    const int64_t p0 = (int64_t)blockIdx.x * tpb * topk;
+    int64_t p1 = p0 + (int64_t)tpb * topk;
+    const int64_t pend = (int64_t)tokens * topk;
+    if (p1 > pend) p1 = pend;
+    for (int64_t i = p0 + threadIdx.x; i < p1; i += blockDim.x) {
+        int64_t e = (int64_t)idx[i];
+        if (e >= 0 && e < experts) atomicAdd(&hist[e], 1);
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) scratch[(int64_t)blockIdx.x * experts + e] = hist[e];
+}
+
+template <typename IdxT>
+__global__ void __launch_bounds__(ZB_LAYOUT_THREADS)
+layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int experts, int ranks, int tpb, int nbits,
+                   const int32_t *__restrict__ scratch, int32_t *__restrict__ send_token_idx,
+                   int32_t *__restrict__ tokens_per_rank)
+{
+    __shared__ int32_t run[ZB_MAX_EXPERTS];
+    __shared__ int32_t rcnt[ZB_MAX_EXPERTS];
+    const int b = blockIdx.x;
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+        int32_t s = 0;
+        for (int bb = 0; bb < b; ++bb) s += scratch[(int64_t)bb * experts + e];
+        run[e] = s;
+    }
+    for (int r = threadIdx.x; r < ranks; r += blockDim.x) rcnt[r] = 0;
+    __syncthreads();
+
+    const int tok0 = b * tpb;
+    int tok1 = tok0 + tpb;
+    if (tok1 > tokens) tok1 = tokens;
+    const int64_t p0 = (int64_t)tok0 * topk, p1 = (int64_t)tok1 * topk;
+    const int np = (int)(p1 - p0);
+    const int iters = (np + ZB_LAYOUT_THREADS - 1) / ZB_LAYOUT_THREADS;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+
+    for (int it = 0; it < iters; ++it) {
+        const int64_t i = p0 + (int64_t)it * ZB_LAYOUT_THREADS + threadIdx.x;
+        int64_t e64 = (i < p1) ? (int64_t)idx[i] : -1;
+        const bool valid = (e64 >= 0 && e64 < experts);
+        const int e = valid ? (int)e64 : 0;
+        uint64_t peers = __ballot(valid);
+        for (int bit = 0; bit < nbits; ++bit) {
+            const bool one = (e >> bit) & 1;
+            const uint64_t bal = __ballot(valid && one);
+            peers &= one ? bal : ~bal;
+        }
+        const int before = __popcll(peers & lt_mask);
+        const int group = __popcll(peers);
+        const bool last = valid && ((peers >> lane) >> 1) == 0; /* highest lane of its group */
+        for (int w = 0; w < ZB_LAYOUT_THREADS / 64; ++w) {
+            if (wave == w && valid) {
+                const int32_t basev = run[e];
+                send_token_idx[i] = basev + before;
+                if (last) run[e] = basev + group;
+            }
+            __syncthreads();
+        }
+        if (!valid && i < p1) send_token_idx[i] = -1;
+    }
+
+    /* tokens per rank: one count per (token, rank) no matter how many of the token's picks land there */
+    if (tokens_per_rank) {
+        const int e_loc = experts / ranks;
+        for (int t = tok0 + threadIdx.x; t < tok1; t += blockDim.x) {
+            for (int k = 0; k < topk; ++k) {
+                int64_t e = (int64_t)idx[(int64_t)t * topk + k];
+                if (e < 0 || e >= experts) continue;
+                const int r = (int)(e / e_loc);
+                bool first = true;
+                for (int k2 = 0; k2 < k; ++k2) {
+                    int64_t e2 = (int64_t)idx[(int64_t)t * topk + k2];
+                    if (e2 >= 0 && e2 < experts && (int)(e2 / e_loc) == r) first = false;
+                }
+                if (first) atomicAdd(&rcnt[r], 1);
+            }
+        }
+        __syncthreads();
+        for (int r = threadIdx.x; r < ranks; r += blockDim.x)
+            if (rcnt[r]) atomicAdd(&tokens_per_rank[r], rcnt[r]);
+    }
+}
+
+/*
+ * One block: totals per expert from the per-block histograms (or from a
+ * ready histogram when nblk == 0), then an inclusive scan over experts.
+ * Every output pointer may be null.
+ */
+__global__ void __launch_bounds__(ZB_MAX_EXPERTS)
+layout_scan_kernel(const int32_t *__restrict__ hist, int nblk, int experts, int topk, int token_nums_type,
+                   int32_t *__restrict__ counts_i32, int32_t *__restrict__ excl_i32, int32_t *__restrict__ incl_i32,
+                   int32_t *__restrict__ row_off /* [E+1] */, int64_t *__restrict__ counts_i64,
+                   int64_t *__restrict__ nums_typed, int32_t *__restrict__ total, int32_t *__restrict__ balance)
+{
+    __shared__ int32_t wsum[ZB_MAX_EXPERTS / 64];
+    const int e = threadIdx.x;
+    int32_t c = 0;
+    if (e < experts) {
+        if (nblk == 0) c = hist[e];
+        else for (int b = 0; b < nblk; ++b) c += hist[(int64_t)b * experts + e];
+    }
+    int32_t s = c;
+    const int lane = e & 63, wave = e >> 6;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        int32_t o = __shfl_up(s, off, 64);
+        if (lane >= off) s += o;
+    }
+    if (lane == 63) wsum[wave] = s;
+    __syncthreads();
+    int32_t add = 0;
+    for (int w = 0; w < wave; ++w) add += wsum[w];
+    s += add;
+    if (e < experts) {
+        if (counts_i32) counts_i32[e] = c;
+        if (excl_i32) excl_i32[e] = s - c;
+        if (incl_i32) incl_i32[e] = s;
+        if (row_off) { row_off[e] = s - c; if (e == experts - 1) row_off[experts] = s; }
+        if (counts_i64) counts_i64[e] = c;
+        if (nums_typed) nums_typed[e] = token_nums_type == 0 ? (int64_t)s : (int64_t)c;
+        if (e == experts - 1) {
+            if (total) *total = s;
+            if (balance) {
+                const int32_t bs = s / topk;
+                balance[0] = bs > 0 ? 0 : -1;
+                balance[1] = bs > 0 ? bs - 1 : -1;
+            }
+        }
+    }
+}
+
+/* ---- router ----------------------------------------------------------------- */
+
+#define ZB_ROUTE_PER_LANE (ZB_MAX_EXPERTS / 64)
+
+__global__ void __launch_bounds__(256)
+topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int topk, int64_t *__restrict__ topk_idx,
+                  float *__restrict__ topk_w)
+{
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (t >= tokens) return; /* whole waves leave together */
+    const float *l = logits + (int64_t)t * experts;
+    float v[ZB_ROUTE_PER_LANE];
+    float mx = -__builtin_inff();
+#pragma unroll
+    for (int j = 0; j < ZB_ROUTE_PER_LANE; ++j) {
+        const int e = j * 64 + lane;
+        v[j] = (e < experts) ? l[e] : -__builtin_inff();
+        mx = fmaxf(mx, v[j]);
+    }
+    mx = zb_wave_max(mx);
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < ZB_ROUTE_PER_LANE; ++j) {
+        const int e = j * 64 + lane;
+        if (e < experts) sum += zb_expf(v[j] - mx);
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+
+    uint32_t used = 0; /* bit j: this lane's j-th logit was picked */
+    float wsum = 0.0f;
+    float myw = 0.0f;  /* lane k keeps the k-th weight (topk <= 32) */
+    int myidx = 0;
+    for (int k = 0; k < topk; ++k) {
+        float best = -__builtin_inff();
+        int bidx = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < ZB_ROUTE_PER_LANE; ++j) {
+            const int e = j * 64 + lane;
+            if (e < experts && !((used >> j) & 1u)) {
+                if (bidx == 0x7fffffff || v[j] > best) { best = v[j]; bidx = e; }
+            }
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ob = __shfl_xor(best, off, 64);
+            const int oi = __shfl_xor(bidx, off, 64);
+            const bool take = (oi != 0x7fffffff) && (bidx == 0x7fffffff || ob > best || (ob == best && oi < bidx));
+            if (take) { best = ob; bidx = oi; }
+        }
+        if ((bidx & 63) == lane) used |= 1u << (bidx >> 6);
+        const float p = zb_expf(best - mx) / sum;
+        wsum += p;
+        if (lane == k) { myw = p; myidx = bidx; }
+    }
+    if (lane < topk) {
+        topk_idx[(int64_t)t * topk + lane] = myidx;
+        topk_w[(int64_t)t * topk + lane] = myw / wsum;
+    }
+}
+
+inline int ceil_log2(int64_t v)
+{
+    int b = 0;
+    while ((1ll << b) < v) ++b;
+    return b;
+}
+
+} // namespace
+
+/* Used by the other translation units of the library (fused path, low-latency dispatch). */
+int32_t zbalhip_layout_internal(const void *idx, int32_t idx_is_i64, int64_t tokens, int64_t experts, int64_t topk,
+                                int32_t ranks, int32_t *tokens_per_rank, int32_t *send_token_idx, int32_t *scratch,
+                                int max_blocks, int *nblk_out, hipStream_t st)
+{
+    const LayoutPlan p = plan_layout(tokens, topk, max_blocks);
+    const int nbits = ceil_log2(experts);
+    if (idx_is_i64) {
+        layout_hist_kernel<int64_t><<<p.nblk, ZB_LAYOUT_THREADS, 0, st>>>(
+            (const int64_t *)idx, (int)tokens, (int)topk, (int)experts, ranks, p.tokens_per_block, scratch,
+            tokens_per_rank);
+        layout_rank_kernel<int64_t><<<p.nblk, ZB_LAYOUT_THREADS, 0, st>>>(
+            (const int64_t *)idx, (int)tokens, (int)topk, (int)experts, ranks, p.tokens_per_block, nbits, scratch,
+            send_token_idx, tokens_per_rank);
+    } else {
+        layout_hist_kernel<int32_t><<<p.nblk, ZB_LAYOUT_THREADS, 0, st>>>(
+            (const int32_t *)idx, (int)tokens, (int)topk, (int)experts, ranks, p.tokens_per_block, scratch,
+            tokens_per_rank);
+        layout_rank_kernel<int32_t><<<p.nblk, ZB_LAYOUT_THREADS, 0, st>>>(
+            (const int32_t *)idx, (int)tokens, (int)topk, (int)experts, ranks, p.tokens_per_block, nbits, scratch,
+            send_token_idx, tokens_per_rank);
+    }
+    *nblk_out = p.nblk;
+    return zbalhip_check_launch();
+}
+
+int32_t zbalhip_scan_internal(const int32_t *hist, int nblk, int64_t experts, int64_t topk, int32_t token_nums_type,
+                              int32_t *counts_i32, int32_t *excl_i32, int32_t *incl_i32, int32_t *row_off,
+                              int64_t *counts_i64, int64_t *nums_typed, int32_t *total, int32_t *balance,
+                              hipStream_t st)
+{
+    int threads = (int)((experts + 63) / 64 * 64);
+    layout_scan_kernel<<<1, threads, 0, st>>>(hist, nblk, (int)experts, (int)topk, token_nums_type, counts_i32,
+                                              excl_i32, incl_i32, row_off, counts_i64, nums_typed, total, balance);
+    return zbalhip_check_launch();
+}
+
+static bool layout_args_ok(int64_t tokens, int64_t experts, int64_t topk)
+{
+    return tokens >= 0 && tokens <= 0x7fffffff / (topk > 0 ? topk : 1) && experts > 0 && experts <= ZB_MAX_EXPERTS &&
+           topk > 0;
+}
+
+extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64_t experts, int64_t topk,
+                                      int64_t *topk_idx, float *topk_w, void *stream)
+{
+    if (!logits || !topk_idx || !topk_w || tokens < 0 || experts <= 0 || experts > ZB_MAX_EXPERTS || topk <= 0 ||
+        topk > 32 || topk > experts)
+        return ZBALHIP_INVALID;
+    if (tokens == 0) return ZBALHIP_OK;
+    const int wpb = 4;
+    const int64_t blocks = (tokens + wpb - 1) / wpb;
+    topk_route_kernel<<<(unsigned)blocks, wpb * 64, 0, (hipStream_t)stream>>>(logits, (int)tokens, (int)experts,
+                                                                           (int)topk, topk_idx, topk_w);
+    return zbalhip_check_launch();
+}
+
+extern "C" int32_t zbalhip_dispatch_layout(const void *topk_idx, int32_t idx_is_i64, int64_t tokens, int64_t experts,
+                                           int64_t topk, int32_t ranks, int32_t *tokens_per_rank,
+                                           int32_t *tokens_per_expert, int32_t *send_token_idx, int32_t *scratch,
+                                           void *stream)
+{
+    if (!topk_idx || !tokens_per_rank || !tokens_per_expert || !send_token_idx || !scratch) return ZBALHIP_INVALID;
+    if (!layout_args_ok(tokens, experts, topk) || ranks <= 0 || ranks > experts || experts % ranks != 0)
+        return ZBALHIP_INVALID;
+    int nblk = 0;
+    int32_t rc = zbalhip_layout_internal(topk_idx, idx_is_i64, tokens, experts, topk, ranks, tokens_per_rank,
+                                         send_token_idx, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, &nblk,
+                                         (hipStream_t)stream);
+    if (rc != ZBALHIP_OK) return rc;
+    return zbalhip_scan_internal(scratch, nblk, experts, topk, 1, tokens_per_expert, nullptr, nullptr, nullptr, nullptr,
+                                 nullptr, nullptr, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int32_t zbalhip_dispatch_notify(const int32_t *tokens_per_expert, int64_t experts, int64_t topk,
+                                           int32_t *recv_data, int32_t *put_offset, int32_t *total_recv,
+                                           int64_t *recv_tokens_per_expert, int32_t *balance_matrix, void *stream)
+{
+    if (!tokens_per_expert || !recv_data || !put_offset || !total_recv || !recv_tokens_per_expert || !balance_matrix)
+        return ZBALHIP_INVALID;
+    if (experts <= 0 || experts > ZB_MAX_EXPERTS || topk <= 0) return ZBALHIP_INVALID;
+    return zbalhip_scan_internal(tokens_per_expert, 0, experts, topk, 1, recv_data, put_offset, nullptr, nullptr,
+                                 recv_tokens_per_expert, nullptr, total_recv, balance_matrix, (hipStream_t)stream);
+}

@@ -1,0 +1,75 @@
+/*
+ * Weight pre-pack: the logical [E, K, N] byte matrix (N contiguous) becomes
+ * [E, N, K] with K contiguous, the order in which the grouped GEMM streams
+ * its B operand; optionally two int4 values are packed per byte. A one-time
+ * step per weight tensor (64x64 tiles transposed through LDS).
+ */
+#include "zbal_device.h"
+#include "zbal_hip_kernels.h"
+
+namespace {
+
+constexpr int kTile = 64;
+
+__global__ void __launch_bounds__(256)
+transpose_bytes_kernel(const uint8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
+{
+    __shared__ uint8_t tile[kTile][kTile + 4];
+    const int64_t e = blockIdx.z;
+    const int64_t k0 = (int64_t)blockIdx.y * kTile, n0 = (int64_t)blockIdx.x * kTile;
+    const uint8_t *s = src + e * K * N;
+    uint8_t *d = dst + e * K * N;
+    for (int i = threadIdx.x; i < kTile * kTile; i += blockDim.x) {
+        const int kk = i / kTile, nn = i % kTile;
+        if (k0 + kk < K && n0 + nn < N) tile[kk][nn] = s[(k0 + kk) * N + n0 + nn];
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < kTile * kTile; i += blockDim.x) {
+        const int nn = i / kTile, kk = i % kTile;
+        if (k0 + kk < K && n0 + nn < N) d[(n0 + nn) * K + k0 + kk] = tile[kk][nn];
+    }
+}
+
+/*
+ * int8 values in [-8,7], [E,K,N] -> [E,N,K/2] bytes. Within every group of 8 consecutive k, byte b (0..3)
+ * holds k[b] in its low nibble and k[b+4] in its high nibble, so that the GEMM unpacks a dword into two
+ * dwords of four consecutive k each with one shift and two masks.
+ */
+__global__ void __launch_bounds__(256)
+transpose_pack_int4_kernel(const int8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
+{
+    __shared__ int8_t tile[kTile][kTile + 4];
+    const int64_t e = blockIdx.z;
+    const int64_t k0 = (int64_t)blockIdx.y * kTile, n0 = (int64_t)blockIdx.x * kTile;
+    const int8_t *s = src + e * K * N;
+    uint8_t *d = dst + e * (K / 2) * N;
+    for (int i = threadIdx.x; i < kTile * kTile; i += blockDim.x) {
+        const int kk = i / kTile, nn = i % kTile;
+        tile[kk][nn] = (k0 + kk < K && n0 + nn < N) ? s[(k0 + kk) * N + n0 + nn] : (int8_t)0;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < kTile * kTile / 2; i += blockDim.x) {
+        const int nn = i / (kTile / 2), kp = i % (kTile / 2);
+        const int kl = (kp / 4) * 8 + (kp % 4); /* k of the low nibble; the high nibble is kl + 4 */
+        if (k0 + kl + 4 < K && n0 + nn < N) {
+            const uint32_t lo = (uint32_t)tile[kl][nn] & 0xfu, hi = (uint32_t)tile[kl + 4][nn] & 0xfu;
+            d[(n0 + nn) * (K / 2) + (k0 / 2) + kp] = (uint8_t)(lo | (hi << 4));
+        }
+    }
+}
+
+} // namespace
+
+extern "C" int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int64_t k, int64_t n, int32_t to_int4,
+                                          void *dst, void *stream)
+{
+    if (!src || !dst || src == dst || experts <= 0 || k <= 0 || n <= 0) return ZBALHIP_INVALID;
+    if (to_int4 && (k % 8) != 0) return ZBALHIP_INVALID;
+    if (experts > 65535 || (k + kTile - 1) / kTile > 65535) return ZBALHIP_INVALID;
+    dim3 grid((unsigned)((n + kTile - 1) / kTile), (unsigned)((k + kTile - 1) / kTile), (unsigned)experts);
+    if (to_int4)
+        transpose_pack_int4_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const int8_t *)src, k, n, (uint8_t *)dst);
+    else
+        transpose_bytes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t *)src, k, n, (uint8_t *)dst);
+    return zbalhip_check_launch();
+}

@@ -1,0 +1,162 @@
+/*
+ * Device-side helpers shared by the gfx950 kernels: scalar format
+ * conversions, the fixed expf used by the SwiGLU epilogue, wave64 reductions
+ * and the launch-error plumbing of the C ABI.
+ *
+ * The kernels are compiled with -ffp-contract=off: a product followed by a
+ * sum rounds twice unless written as __builtin_fmaf().
+ */
+#ifndef ZBAL_DEVICE_H_
+#define ZBAL_DEVICE_H_
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define ZBALHIP_OK 0
+#define ZBALHIP_INVALID (-2)
+#define ZBALHIP_RT_ERROR (-11)
+
+/* zbal_datatype_t values used by the kernels */
+#define ZDT_INT8 0
+#define ZDT_INT16 1
+#define ZDT_INT32 2
+#define ZDT_INT64 3
+#define ZDT_FP16 6
+#define ZDT_FP32 7
+#define ZDT_BF16 8
+
+#define ZBAL_WAVE 64
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
+typedef int32_t i32x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+static inline int32_t zbalhip_check_launch()
+{
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? ZBALHIP_OK : ZBALHIP_RT_ERROR;
+}
+
+/* ---- scalar formats ------------------------------------------------------ */
+
+__device__ __forceinline__ float zb_bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
+
+__device__ __forceinline__ uint32_t zb_f32_to_bf16(float f)
+{
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+__device__ __forceinline__ float zb_fp16_to_f32(uint32_t h)
+{
+    _Float16 v;
+    uint16_t s = (uint16_t)h;
+    __builtin_memcpy(&v, &s, 2);
+    return (float)v;
+}
+
+__device__ __forceinline__ uint32_t zb_f32_to_fp16(float f)
+{
+    /*
+     * The empty asm keeps the compiler from folding a preceding fp32 multiply into v_fma_mixlo_f16, which
+     * rounds the exact product straight to fp16; the result must be the fp32-rounded product rounded again.
+     */
+    asm volatile("" : "+v"(f));
+    _Float16 v = (_Float16)f; /* v_cvt_f16_f32: round to nearest even */
+    uint16_t s;
+    __builtin_memcpy(&s, &v, 2);
+    return s;
+}
+
+template <int DT> __device__ __forceinline__ float zb_half_to_f32(uint32_t h)
+{
+    if constexpr (DT == ZDT_FP16) return zb_fp16_to_f32(h);
+    else return zb_bf16_to_f32(h);
+}
+
+template <int DT> __device__ __forceinline__ uint32_t zb_f32_to_half(float f)
+{
+    if constexpr (DT == ZDT_FP16) return zb_f32_to_fp16(f);
+    else return zb_f32_to_bf16(f);
+}
+
+/* two floats -> two e4m3 codes in the low 16 bits (v_cvt_pk_fp8_f32, OCP format on gfx950); inputs pre-clamped */
+__device__ __forceinline__ uint32_t zb_cvt_pk_e4m3(float a, float b)
+{
+    a = fminf(fmaxf(a, -448.0f), 448.0f);
+    b = fminf(fmaxf(b, -448.0f), 448.0f);
+    return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+}
+
+/* round-half-even to int, clamped to int8 */
+__device__ __forceinline__ int32_t zb_rint_i8(float v)
+{
+    float r = __builtin_rintf(v);
+    r = fminf(fmaxf(r, -128.0f), 127.0f);
+    return (int32_t)r;
+}
+
+/*
+ * exp() of the SwiGLU epilogue: Cody-Waite reduction by ln2, a degree-6
+ * polynomial in fmaf form and scaling by two exact powers of two. The same
+ * operation sequence is what the CPU checker evaluates, so both sides agree
+ * bit for bit (the hardware v_exp_f32 is an approximation and would not).
+ */
+__device__ __forceinline__ float zb_expf(float x)
+{
+    if (!(x == x)) return x;
+    if (x > 88.72284f) return __builtin_inff();
+    if (x < -103.97208f) return 0.0f;
+    float n = __builtin_rintf(x * 1.44269504088896341f);
+    float r = __builtin_fmaf(n, -0.693145751953125f, x);
+    r = __builtin_fmaf(n, -1.42860682030941723e-06f, r);
+    float p = 1.3888889e-03f;
+    p = __builtin_fmaf(p, r, 8.3333333e-03f);
+    p = __builtin_fmaf(p, r, 4.1666668e-02f);
+    p = __builtin_fmaf(p, r, 1.6666667e-01f);
+    p = __builtin_fmaf(p, r, 0.5f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    p = __builtin_fmaf(p, r, 1.0f);
+    int ni = (int)n;
+    int n1 = ni / 2, n2 = ni - n1;
+    float s1 = __uint_as_float((uint32_t)(n1 + 127) << 23);
+    float s2 = __uint_as_float((uint32_t)(n2 + 127) << 23);
+    return (p * s1) * s2;
+}
+
+/* ---- wave64 reductions ------------------------------------------------------ */
+
+__device__ __forceinline__ float zb_wave_max(float v)
+{
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, ZBAL_WAVE));
+    return v;
+}
+
+/* max over groups of 2^LOG2 consecutive lanes */
+template <int LOG2> __device__ __forceinline__ float zb_group_max(float v)
+{
+#pragma unroll
+    for (int off = (1 << LOG2) >> 1; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, ZBAL_WAVE));
+    return v;
+}
+
+/* block-wide max through LDS; `red` holds one float per wave; all threads receive the result */
+__device__ __forceinline__ float zb_block_max(float v, float *red)
+{
+    v = zb_wave_max(v);
+    const int lane = threadIdx.x & (ZBAL_WAVE - 1), wave = threadIdx.x / ZBAL_WAVE;
+    const int nwaves = (blockDim.x + ZBAL_WAVE - 1) / ZBAL_WAVE;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int i = 1; i < nwaves; ++i) r = fmaxf(r, red[i]);
+    return r;
+}
+
+#endif /* ZBAL_DEVICE_H_ */

@@ -1,0 +1,201 @@
+"""Host-side checks that need no GPU: the C ABI library loads and exports every
+declared symbol, struct layouts match the reference's, validation and the
+communicator lifecycle return the reference's codes (exercised on the
+do-nothing backend, as the reference's own unit tests do)."""
+import ctypes
+import os
+import re
+import subprocess
+
+import pytest
+
+from memfabric_hybrid_amd import capi
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+INC = os.path.join(ROOT, "include")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return capi.load()
+
+
+def declared_symbols():
+    names = set()
+    for f in os.listdir(INC):
+        text = open(os.path.join(INC, f)).read()
+        text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+        names |= set(re.findall(r"\b(zbal(?:hip)?_\w+)\s*\(", text))
+    return names
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    decl = declared_symbols()
+    assert len(decl) >= 38
+    for name in decl:
+        assert hasattr(lib, name), "library does not export %s" % name
+    assert decl == set(capi.SIGNATURES), decl ^ set(capi.SIGNATURES)
+
+
+def test_headers_compile_as_c_and_cpp_and_struct_sizes(tmp_path):
+    src = tmp_path / "t.c"
+    src.write_text('#include "zbal.h"\n#include "zbal_hip_kernels.h"\n#include <stdio.h>\n'
+                   'int main(void){printf("%zu %zu %zu %zu %zu\\n", sizeof(zbal_tensor_info_t),'
+                   'sizeof(zbal_comm_options_t), sizeof(zbal_comm_property_t), sizeof(zbal_bootstrap_options_t),'
+                   '__builtin_offsetof(zbal_tensor_info_t, shape));return 0;}\n')
+    exe = tmp_path / "t"
+    subprocess.check_call(["gcc", "-I", INC, str(src), "-o", str(exe)])
+    out = subprocess.check_output([str(exe)]).decode().split()
+    # reference zbal_def.h:141-147 measures 72 bytes with gcc on x86-64 (its comment says 64)
+    assert int(out[0]) == 72 == ctypes.sizeof(capi.TensorInfo)
+    assert int(out[1]) == ctypes.sizeof(capi.CommOptions)
+    assert int(out[2]) == ctypes.sizeof(capi.CommProperty)
+    assert int(out[3]) == ctypes.sizeof(capi.BootstrapOptions)
+    assert int(out[4]) == 16 == capi.TensorInfo.shape.offset
+    subprocess.check_call(["g++", "-std=c++17", "-fsyntax-only", "-x", "c++", "-I", INC, os.path.join(INC, "zbal.h")])
+
+
+def test_enum_values_match_reference():
+    assert (capi.DT_INT8, capi.DT_FP16, capi.DT_FP32, capi.DT_BF16, capi.DT_UINT32) == (0, 6, 7, 8, 11)
+    assert (capi.REDUCE_PROD, capi.REDUCE_SUM, capi.REDUCE_MAX, capi.REDUCE_MIN) == (0, 1, 2, 3)
+    assert (capi.NO_QUANT, capi.QUANT_INT8) == (0, 1)
+
+
+def test_version_logger_and_last_error(lib):
+    assert b"zbal" in lib.zbal_version()
+    assert lib.zbal_set_logger_level(7) == capi.Z_INVALID_PARAM
+    assert lib.zbal_set_logger_level(3) == 0
+    seen = []
+    CB = ctypes.CFUNCTYPE(None, ctypes.c_int, ctypes.c_char_p)
+    cb = CB(lambda lvl, msg: seen.append((lvl, msg)))
+    lib.zbal_set_logger(ctypes.cast(cb, ctypes.c_void_p))
+    assert lib.zbal_comm_destroy(None, 0) == capi.Z_INVALID_PARAM
+    assert seen and seen[-1][0] == 3 and b"comm is null" in seen[-1][1]
+    assert b"comm is null" in lib.zbal_get_last_error_msg()
+    assert b"comm is null" in lib.zbal_get_and_clear_last_error_msg()
+    assert lib.zbal_get_last_error_msg() == b""
+    lib.zbal_set_logger(None)
+
+
+@pytest.fixture
+def host_world(lib):
+    """Bootstrap without touching a device (flags bit 0) and tear down afterwards."""
+    opts = capi.BootstrapOptions()
+    assert lib.zbal_bootstrap_options_init(ctypes.byref(opts)) == 0
+    opts.flags = 1
+    opts.worldSize = 8
+    opts.rankId = 3
+    assert lib.zbal_bootstrap(ctypes.byref(opts), None) == 0
+    yield lib
+    lib.zbal_comm_destroy_all(0)
+    assert lib.zbal_unbootstrap(0) == 0
+
+
+def make_comm(lib, name, world, size, rank, backend=capi.BACKEND_DUMMY):
+    co = capi.CommOptions(name=name, backendType=backend, isWorldGroup=world, groupSize=size, groupRankId=rank)
+    comm = ctypes.c_void_p()
+    rc = lib.zbal_comm_create(ctypes.byref(co), ctypes.byref(comm))
+    return rc, comm
+
+
+def test_create_needs_bootstrap(lib):
+    lib.zbal_set_logger_level(3)
+    rc, _ = make_comm(lib, b"w", 1, 1, 0)
+    assert rc == capi.Z_NOT_BOOTSTRAPPED
+    assert lib.zbal_unbootstrap(0) == -14
+
+
+def test_communicator_lifecycle(host_world):
+    lib = host_world
+    assert lib.zbal_bootstrap(ctypes.byref(capi.BootstrapOptions(worldSize=1)), None) == -13   # already bootstrapped
+    assert lib.zbal_comm_get_global() is None
+    rc, _ = make_comm(lib, b"sub", 0, 4, 1)
+    assert rc == capi.Z_CREATE_COMM_FAILED              # world group must come first
+    rc, _ = make_comm(lib, b"world", 1, 4, 1)
+    assert rc == capi.Z_NOT_BOOTSTRAPPED                # size differs from the bootstrap's world size
+    rc, world = make_comm(lib, b"world", 1, 8, 3)
+    assert rc == 0 and lib.zbal_comm_get_global() == world.value
+    rc, _ = make_comm(lib, b"world2", 1, 8, 3)
+    assert rc == capi.Z_CREATE_COMM_FAILED              # only one world group
+    rc, sub = make_comm(lib, b"sub", 0, 4, 1)
+    assert rc == 0
+    rc, _ = make_comm(lib, b"sub", 0, 4, 1)
+    assert rc == capi.Z_CREATE_COMM_FAILED              # duplicate name
+    rc, _ = make_comm(lib, b"big", 0, 16, 1)
+    assert rc == capi.Z_NOT_BOOTSTRAPPED                # bigger than the world
+    rc, _ = make_comm(lib, b"", 0, 4, 1)
+    assert rc == capi.Z_INVALID_PARAM
+    rc, _ = make_comm(lib, b"x" * 128, 0, 4, 1)
+    assert rc == capi.Z_INVALID_PARAM
+    assert lib.zbal_comm_get_by_name(b"sub") == sub.value
+    assert lib.zbal_comm_get_by_name(b"nope") is None
+    prop = capi.CommProperty()
+    assert lib.zbal_comm_get_property(sub, ctypes.byref(prop)) == 0
+    assert (prop.groupSize, prop.groupRankId, prop.isWorldGroup, prop.name) == (4, 1, 0, b"sub")
+    assert lib.zbal_comm_get_property(ctypes.c_void_p(0x1234), ctypes.byref(prop)) == capi.Z_COMM_NOT_EXIST_BY_HANDLE
+    assert lib.zbal_comm_destroy(world, 0) == capi.Z_COMM_DESTROY_GLOBAL_LAST
+    assert lib.zbal_comm_destroy(ctypes.c_void_p(0x1234), 0) == 0     # unknown handle: not an error
+    assert lib.zbal_comm_destroy(sub, 0) == 0
+    assert lib.zbal_comm_get_by_name(b"sub") is None
+    assert lib.zbal_comm_destroy(world, 0) == 0
+    assert lib.zbal_comm_get_global() is None
+
+
+def test_operator_validation_codes(host_world):
+    """The null / range checks of reference zbal_operations.cpp and test_zbal_operations.cpp:166-213, 408-455."""
+    lib = host_world
+    rc, world = make_comm(lib, b"world", 1, 8, 3)
+    assert rc == 0
+    buf = ctypes.create_string_buffer(64)
+    p = ctypes.cast(buf, ctypes.c_void_p)
+    # null send buffer is a silent success
+    assert lib.zbal_all_reduce(None, p, p, 4, capi.DT_FP32, capi.REDUCE_SUM, world, None) == 0
+    assert lib.zbal_reduce_scatter(None, p, 4, capi.DT_FP32, capi.REDUCE_SUM, world, None) == 0
+    assert lib.zbal_all_reduce(p, None, p, 4, capi.DT_FP32, capi.REDUCE_SUM, world, None) == -2
+    assert lib.zbal_all_reduce(p, p, p, 0, capi.DT_FP32, capi.REDUCE_SUM, world, None) == -2
+    assert lib.zbal_all_reduce(p, p, p, 4, 99, capi.REDUCE_SUM, world, None) == -2
+    assert lib.zbal_all_reduce(p, p, p, 4, capi.DT_FP32, 9, world, None) == -2
+    assert lib.zbal_all_reduce(p, p, p, 4, capi.DT_FP32, capi.REDUCE_SUM, None, None) == -2
+    assert lib.zbal_all_reduce(p, p, None, 4, capi.DT_FP32, capi.REDUCE_SUM, world, None) == -2
+    assert lib.zbal_all_reduce(p, p, p, 4, capi.DT_FP32, capi.REDUCE_SUM, world, None) == 0      # dummy backend
+    assert lib.zbal_reduce_scatter(p, p, 0, capi.DT_FP32, capi.REDUCE_SUM, world, None) == -2
+    ti = capi.TensorInfo()
+    t = ctypes.byref(ti)
+    assert lib.zbal_dispatch_normal_layout(None, 4, 8, 2, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal_layout(t, -1, 8, 2, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal_layout(t, 4, 0, 2, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal_layout(t, 4, 8, 0, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal_layout(t, 4, 8, 2, t, t, t, t, None, None, 0) == -2           # reference dereferences null here
+    assert lib.zbal_dispatch_normal_layout(t, 4, 8, 2, t, t, t, t, ctypes.c_void_p(0x40), None, 0) == -2
+    assert lib.zbal_dispatch_normal_layout(t, 4, 8, 2, t, t, t, t, world, None, 0) == 0
+    assert lib.zbal_dispatch_normal_notify(t, 0, 2, t, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal_notify(t, 8, 2, t, t, None, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal(t, t, t, t, t, 0, 0, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_normal(t, t, t, t, t, 8, 0, t, None, world, None, 0) == -2
+    assert lib.zbal_combine_normal(t, t, t, t, t, t, 0, t, world, None, 0) == -2
+    assert lib.zbal_combine_normal(t, t, None, t, t, t, 8, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_low_latency(t, t, 0, 0, 0, 0, 0, 0, 1, t, t, t, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_low_latency(t, t, 8, -1, 0, 0, 0, 0, 1, t, t, t, t, t, t, t, world, None, 0) == -2
+    assert lib.zbal_dispatch_low_latency(t, t, 8, 0, 0, 0, 0, 0, 1, t, t, t, t, t, t, None, world, None, 0) == -2
+    assert lib.zbal_combine_low_latency(t, t, t, t, t, None, 8, world, None, 0) == -2
+    assert lib.zbal_combine_low_latency(t, t, t, t, t, t, 0, world, None, 0) == -2
+    fused = [t] * 7 + [None] * 7 + [t, None, t, t]
+    assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 256, 0, 0, world, None, 0) == 0
+    assert lib.zbal_fused_deep_moe(*fused, 0, 0, 0, 256, 0, 0, world, None, 0) == -2
+    assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 0, 0, 0, world, None, 0) == -2
+    assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 256, 0, 1, world, None, 0) == -2              # tensor list
+    bad = list(fused); bad[17] = None
+    assert lib.zbal_fused_deep_moe(*bad, 8, 0, 0, 256, 0, 0, world, None, 0) == -2                # workspace
+    assert lib.zbal_comm_register_peer_window(world, 9, p, 64) == -2
+    assert lib.zbal_comm_register_peer_window(world, 1, None, 64) == -2
+    assert lib.zbal_comm_register_peer_window(world, 1, p, 64) in (0, -2)   # alignment of a host buffer varies
+
+
+def test_fused_workspace_size_is_monotonic(lib):
+    f = lib.zbal_fused_deep_moe_workspace_size
+    assert f(0, 7168, 8, 32, 4096, 2) > 0
+    a, b = f(128, 7168, 8, 32, 4096, 0), f(256, 7168, 8, 32, 4096, 0)
+    assert 0 < a < b
+    assert f(128, 7168, 8, 32, 4000, 0) == 0 and f(128, 100, 8, 32, 4096, 0) == 0 and f(128, 7168, 8, 32, 4096, 9) == 0
+    # W8A8 keeps an fp32 SwiGLU scratch that the fp8 mode does not need
+    assert f(128, 7168, 8, 32, 4096, 2) < f(128, 7168, 8, 32, 4096, 0)

@@ -1,0 +1,267 @@
+"""Parity of the HIP path against the CPU oracle, called through the C ABI on identical seeded inputs.
+Integer outputs (indices, offsets, permutation, quantised bytes, scales) must match bit for bit; bf16
+GEMM / combine outputs within max relative error 2e-2; fp32 reductions within 1e-6."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from memfabric_hybrid_amd import capi
+from memfabric_hybrid_amd.buffer import Buffer
+from oracle import oracle as zo
+from zbal_testlib import bf16_normal, calc_diff, dev, distinct_topk, host, max_rel_err, rng
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def buf():
+    b = Buffer()
+    yield b
+    torch.cuda.synchronize()
+    b.close()
+
+
+# ---- router ---------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("T,E,K", [(256, 8, 2), (300, 32, 8), (64, 128, 8), (17, 256, 6), (5, 1000, 32)])
+def test_router(buf, T, E, K):
+    logits = rng(T + E).standard_normal((T, E)).astype(np.float32)
+    logits[0, :] = 0.5                       # all tied: lowest indices win
+    logits[1, E - 1] = logits[1, 0]          # one tie
+    idx, w = buf.topk_route(dev(logits), K)
+    ridx, rw = zo.topk_route(logits, K)
+    assert np.array_equal(host(idx), ridx)
+    assert np.allclose(host(w), rw, rtol=2e-6, atol=0)     # north star: weights within 1e-6 relative (2 ulp slack)
+
+
+# ---- layout / notify -------------------------------------------------------------------------
+
+@pytest.mark.parametrize("T,K,E", [(256, 2, 8), (4096, 8, 32), (16384, 8, 128), (1, 1, 1), (7, 3, 5), (1000, 6, 256),
+                                    (128, 8, 32)])
+def test_layout_and_notify(buf, T, K, E):
+    idx = rng(T * 31 + E).integers(-1, E + 1, size=(T, K)).astype(np.int64) if T < 2000 else distinct_topk(T, E, K, 3)
+    per_rank, _, per_expert, in_rank, _ = buf.get_dispatch_layout(dev(idx), E)
+    r_rank, r_exp, r_send = zo.dispatch_layout(idx, E, 1)
+    assert np.array_equal(host(per_expert), r_exp)
+    assert np.array_equal(host(per_rank), r_rank)
+    assert np.array_equal(host(buf.send_token_idx), r_send)
+    x = dev(bf16_normal((T, 64), 1))
+    _, _, recv_per_expert, h = buf.dispatch(x, dev(idx), None, per_expert, capi.NO_QUANT)
+    r_recv, r_put, r_total, r_per, r_bal = zo.dispatch_notify(r_exp[None, :], K)
+    assert np.array_equal(host(h["put_offset"]), r_put)
+    assert np.array_equal(host(h["total_recv"]), r_total)
+    assert np.array_equal(host(recv_per_expert), r_per)
+    assert np.array_equal(host(h["balance_matrix"]), r_bal)
+
+
+def test_layout_int32_indices_and_empty_batch(buf):
+    lib = buf.lib
+    E, K = 16, 4
+    idx = distinct_topk(50, E, K, 9).astype(np.int32)
+    t_idx = dev(idx)
+    per_rank = torch.empty(1, dtype=torch.int32, device="cuda")
+    per_exp = torch.empty(E, dtype=torch.int32, device="cuda")
+    send = torch.empty((50, K), dtype=torch.int32, device="cuda")
+    scratch = torch.empty(50 * E, dtype=torch.int32, device="cuda")
+    ti = lambda t: ctypes.byref(capi.tensor_info(t))
+    assert lib.zbal_dispatch_normal_layout(ti(t_idx), 50, E, K, ti(per_rank), ti(per_exp), ti(send), ti(scratch),
+                                           buf.comm, capi.stream_ptr(), 0) == 0
+    r_rank, r_exp, r_send = zo.dispatch_layout(idx.astype(np.int64), E, 1)
+    assert np.array_equal(host(per_exp), r_exp) and np.array_equal(host(send), r_send)
+    # zero tokens: counts are zeroed, nothing else is touched
+    assert lib.zbal_dispatch_normal_layout(ti(t_idx), 0, E, K, ti(per_rank), ti(per_exp), ti(send), ti(scratch),
+                                           buf.comm, capi.stream_ptr(), 0) == 0
+    assert host(per_exp).sum() == 0 and host(per_rank)[0] == 0
+    # too small a scratch tensor is refused, not overrun
+    small = torch.empty(E, dtype=torch.int32, device="cuda")
+    assert lib.zbal_dispatch_normal_layout(ti(t_idx), 50, E, K, ti(per_rank), ti(per_exp), ti(send), ti(small),
+                                           buf.comm, capi.stream_ptr(), 0) == capi.Z_INVALID_PARAM
+
+
+# ---- dispatch (permute + quant) and combine --------------------------------------------------------
+
+def run_dispatch(buf, x16, xdt, idx, E, qmode):
+    tdt = torch.bfloat16 if xdt == zo.DT_BF16 else torch.float16
+    per_rank, _, per_expert, _, _ = buf.get_dispatch_layout(dev(idx), E)
+    recv, scales, _, h = buf.dispatch(dev(x16, tdt), dev(idx), None, per_expert, qmode)
+    _, r_exp, r_send = zo.dispatch_layout(idx, E, 1)
+    put = np.concatenate([[0], np.cumsum(r_exp)[:-1]]).astype(np.int32)
+    rows = int(r_exp.sum())
+    r_dest, r_scale = zo.dispatch_normal(x16, xdt, idx.astype(np.int32), r_send, put, E, qmode, rows)
+    return recv, scales, h, r_dest, r_scale, rows, put, r_send
+
+
+@pytest.mark.parametrize("T,H,K,E", [(256, 1024, 2, 8), (128, 7168, 8, 32), (64, 4096, 8, 128), (33, 128, 3, 4),
+                                      (9, 16384, 2, 4)])
+@pytest.mark.parametrize("qmode", [capi.NO_QUANT, capi.QUANT_INT8, capi.QUANT_FP8_B128])
+def test_dispatch_normal_bit_exact(buf, T, H, K, E, qmode):
+    x = bf16_normal((T, H), T + H)
+    xf = zo.bf16_to_f32(x)
+    xf[0, :] = 0.0                  # all-zero token
+    xf[1 % T, :] = -2.5             # constant token
+    x = zo.f32_to_bf16(xf)
+    idx = distinct_topk(T, E, K, 5)
+    idx[2 % T, 0] = -1              # an invalid pick
+    recv, scales, h, r_dest, r_scale, rows, _, _ = run_dispatch(buf, x, zo.DT_BF16, idx, E, qmode)
+    got = host(recv)[:rows]
+    assert np.array_equal(got.view(r_dest.dtype), r_dest)
+    if qmode != capi.NO_QUANT:
+        assert np.array_equal(host(scales)[:rows].view(np.uint32), r_scale.view(np.uint32))
+
+
+def test_dispatch_fp16_input(buf):
+    T, H, K, E = 40, 512, 4, 16
+    x = zo.f32_to_fp16(rng(8).standard_normal((T, H)).astype(np.float32) * 3)
+    idx = distinct_topk(T, E, K, 6)
+    for qmode in (capi.NO_QUANT, capi.QUANT_INT8, capi.QUANT_FP8_B128):
+        recv, scales, h, r_dest, r_scale, rows, _, _ = run_dispatch(buf, x, zo.DT_FP16, idx, E, qmode)
+        assert np.array_equal(host(recv)[:rows].view(r_dest.dtype), r_dest)
+        if qmode != capi.NO_QUANT:
+            assert np.array_equal(host(scales)[:rows], r_scale)
+
+
+@pytest.mark.parametrize("T,H,K,E", [(256, 2048, 2, 8), (128, 7168, 8, 32), (50, 4096, 8, 128), (3, 64, 1, 2)])
+def test_combine_normal_exact_and_round_trip(buf, T, H, K, E):
+    x = bf16_normal((T, H), 11)
+    idx = distinct_topk(T, E, K, 12)
+    if T > 2:
+        idx[1, K - 1] = -1
+    w = rng(13).uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    recv, _, h, r_dest, _, rows, put, r_send = run_dispatch(buf, x, zo.DT_BF16, idx, E, capi.NO_QUANT)
+    out = buf.combine(recv, h, dev(w))
+    ref = zo.combine(r_dest, zo.DT_BF16, put, w, idx.astype(np.int32), r_send, E)
+    assert np.array_equal(host(out), ref)                         # same operation order: bit exact
+    # the reference's own check (test_normal.py:225-236): identity experts give x * sum of the valid weights
+    wv = np.where((idx >= 0) & (idx < E), w, 0).sum(1, keepdims=True)
+    assert calc_diff(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(x) * wv) < 5e-5
+
+
+def test_combine_fp16(buf):
+    T, H, K, E = 20, 256, 4, 8
+    x = zo.f32_to_fp16(rng(14).standard_normal((T, H)).astype(np.float32))
+    idx = distinct_topk(T, E, K, 15)
+    w = rng(16).uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    recv, _, h, r_dest, _, rows, put, r_send = run_dispatch(buf, x, zo.DT_FP16, idx, E, capi.NO_QUANT)
+    out = buf.combine(recv, h, dev(w))
+    assert np.array_equal(host(out), zo.combine(r_dest, zo.DT_FP16, put, w, idx.astype(np.int32), r_send, E))
+
+
+# ---- low-latency mode ------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("T,H,K,E,zipf", [(128, 7168, 8, 32, 1.2), (1, 7168, 8, 32, None), (80, 4096, 8, 128, None),
+                                           (300, 256, 4, 16, None)])
+@pytest.mark.parametrize("mode", ["bf16", "int8", "fp8"])
+def test_low_latency_dispatch_combine(buf, T, H, K, E, zipf, mode):
+    x = bf16_normal((T, H), 21)
+    if T > 1:
+        x[1, :] = 0                     # all-zero token: q = 0, scale = 0 in this mode
+    idx = distinct_topk(T, E, K, 22, zipf=zipf)
+    w = rng(23).uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    use_fp8, blk, qm = {"bf16": (False, False, 0), "int8": (True, False, 1), "fp8": (True, True, 2)}[mode]
+    recv, scales, count, h = buf.low_latency_dispatch(dev(x), dev(idx), T, E, use_fp8=use_fp8, fp8_block_scale=blk)
+    rows = T * K
+    r_ex, r_sc, r_eidx, r_nums, r_counts = zo.dispatch_low_latency(x, zo.DT_BF16, idx.astype(np.int32), E, qm, rows)
+    assert np.array_equal(host(h["expand_idx"])[:rows].reshape(T, K), r_eidx)
+    assert np.array_equal(host(count), r_nums) and np.array_equal(host(h["ep_recv_count"]), r_counts)
+    assert np.array_equal(host(recv).view(r_ex.dtype), r_ex)
+    if qm:
+        assert np.array_equal(host(scales).view(np.uint32), r_sc.view(np.uint32))
+    if mode == "bf16":
+        out = buf.low_latency_combine(recv, dev(w), h)
+        ref = zo.combine_low_latency(r_ex, zo.DT_BF16, idx.astype(np.int32), r_eidx, r_counts, w, E)
+        assert np.array_equal(host(out), ref)
+        assert calc_diff(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(x) * w.sum(1, keepdims=True)) < 1e-5
+
+
+def test_low_latency_token_nums_type_prefix_sum(buf, monkeypatch):
+    monkeypatch.setenv("MOE_EXPERT_TOKEN_NUMS_TYPE", "0")
+    T, H, K, E = 64, 256, 4, 16
+    idx = distinct_topk(T, E, K, 24)
+    _, _, count, _ = buf.low_latency_dispatch(dev(bf16_normal((T, H), 25)), dev(idx), T, E, use_fp8=False)
+    assert np.array_equal(host(count), np.cumsum(np.bincount(idx.reshape(-1), minlength=E)))
+
+
+# ---- N-buffer reduce ----------------------------------------------------------------------------------
+
+NP_DT = {capi.DT_INT8: np.int8, capi.DT_INT16: np.int16, capi.DT_INT32: np.int32, capi.DT_INT64: np.int64,
+         capi.DT_FP32: np.float32}
+
+
+def make_reduce_inputs(dt, n, N, seed):
+    if dt in NP_DT and dt != capi.DT_FP32:
+        return [rng(seed + p).integers(-100, 100, n).astype(NP_DT[dt]) for p in range(N)]
+    f = [rng(seed + p).uniform(0, 10, n).astype(np.float32) - (3 if p % 2 else 0) for p in range(N)]  # reference: uniform(0,10)
+    if dt == capi.DT_FP32:
+        return f
+    return [zo.f32_to_bf16(a) if dt == capi.DT_BF16 else zo.f32_to_fp16(a) for a in f]
+
+
+@pytest.mark.parametrize("dt", [capi.DT_INT8, capi.DT_INT16, capi.DT_INT32, capi.DT_INT64, capi.DT_FP16, capi.DT_BF16,
+                                capi.DT_FP32])
+@pytest.mark.parametrize("op", [capi.REDUCE_SUM, capi.REDUCE_MAX, capi.REDUCE_MIN, capi.REDUCE_PROD])
+def test_reduce_kernel_all_types(buf, dt, op):
+    lib = buf.lib
+    for N, n in ((8, 6 * 2 ** 10 + 5), (3, 1000), (1, 77), (16, 4096), (5, 3)):
+        ins = make_reduce_inputs(dt, n, N, 100 + N)
+        tdt = {capi.DT_BF16: torch.bfloat16, capi.DT_FP16: torch.float16}.get(dt)
+        d_in = [dev(a, tdt) for a in ins]
+        out = torch.empty_like(d_in[0])
+        arr = (ctypes.c_void_p * N)(*[t.data_ptr() for t in d_in])
+        assert lib.zbalhip_reduce(arr, N, n, dt, op, out.data_ptr(), capi.stream_ptr()) == 0
+        ref = zo.reduce(ins, dt, op)
+        assert np.array_equal(host(out), ref), (N, n)
+
+
+def test_reduce_scatter_and_all_reduce_over_peer_windows(buf):
+    """cfg4 shape in miniature: 8 'ranks' as local windows, this rank reduces its slice of every peer's buffer."""
+    from memfabric_hybrid_amd.buffer import create_group, destroy_group
+    lib = buf.lib
+    R, me, n = 8, 5, 6 * 2 ** 12
+    comm = create_group("rs8", R, me)
+    try:
+        for dt, tdt in ((capi.DT_BF16, torch.bfloat16), (capi.DT_FP32, None)):
+            ins = make_reduce_inputs(dt, R * n, R, 300)
+            wins = [dev(a, tdt) for a in ins]
+            esz = wins[0].element_size()
+            recv = torch.empty(n, dtype=wins[0].dtype, device="cuda")
+            if dt == capi.DT_BF16:   # without windows the send buffer cannot be translated
+                assert lib.zbal_reduce_scatter(wins[me].data_ptr(), recv.data_ptr(), n, dt, capi.REDUCE_SUM, comm,
+                                               capi.stream_ptr()) == capi.Z_INVALID_PARAM
+            for r in range(R):
+                assert lib.zbal_comm_register_peer_window(comm, r, wins[r].data_ptr(), R * n * esz) == 0
+            assert lib.zbal_reduce_scatter(wins[me].data_ptr(), recv.data_ptr(), n, dt, capi.REDUCE_SUM, comm,
+                                           capi.stream_ptr()) == 0
+            ref = zo.reduce([a[me * n:(me + 1) * n].copy() for a in ins], dt, capi.REDUCE_SUM)
+            assert np.array_equal(host(recv), ref)
+            full = torch.empty(R * n, dtype=wins[0].dtype, device="cuda")
+            tmp = torch.empty(n, dtype=wins[0].dtype, device="cuda")
+            assert lib.zbal_all_reduce(wins[me].data_ptr(), full.data_ptr(), tmp.data_ptr(), R * n, dt, capi.REDUCE_SUM,
+                                       comm, capi.stream_ptr()) == 0
+            assert np.array_equal(host(full), zo.reduce(ins, dt, capi.REDUCE_SUM))
+            if dt == capi.DT_FP32:     # north star: fp32 within 1e-6 relative of the exact sum
+                exact = np.sum(np.stack(ins).astype(np.float64), 0)
+                assert np.allclose(host(full), exact, rtol=1e-6, atol=1e-6)
+            # a send buffer outside this rank's window is refused
+            assert lib.zbal_reduce_scatter(recv.data_ptr(), recv.data_ptr(), n, dt, capi.REDUCE_SUM, comm,
+                                           capi.stream_ptr()) == capi.Z_INVALID_PARAM
+            torch.cuda.synchronize()
+    finally:
+        torch.cuda.synchronize()
+        destroy_group(comm)
+
+
+# ---- weight pre-pack --------------------------------------------------------------------------------------
+
+def test_weight_prepack(buf):
+    E, K, N = 3, 200, 136
+    w = rng(40).integers(-128, 128, (E, K, N)).astype(np.int8)
+    packed = buf.prepack_weight(dev(w))
+    assert np.array_equal(host(packed), np.ascontiguousarray(w.transpose(0, 2, 1)))
+    K = 256
+    w4 = rng(41).integers(-8, 8, (E, K, N)).astype(np.int8)
+    p4 = host(buf.prepack_weight(dev(w4), int4=True))
+    wt = w4.transpose(0, 2, 1).reshape(E, N, K // 8, 8)
+    want = ((wt[..., :4] & 0xf) | ((wt[..., 4:] & 0xf) << 4)).astype(np.uint8).reshape(E, N, K // 2)
+    assert np.array_equal(p4, want)

@@ -1,0 +1,59 @@
+"""Shared helpers of the GPU parity tests: seeded inputs as numpy arrays, copies to and from
+the device, and the comparison metrics (the reference's calc_diff among them)."""
+import numpy as np
+import torch
+
+from oracle import oracle as zo
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def dev(a, dtype=None):
+    """numpy -> cuda tensor. uint16 arrays carry bf16/fp16 bit patterns (pass dtype), uint8 may carry e4m3."""
+    t = torch.from_numpy(np.ascontiguousarray(a))
+    if a.dtype == np.uint16:
+        t = t.view(torch.int16).view(dtype or torch.bfloat16)
+    elif dtype is not None and a.dtype == np.uint8:
+        t = t.view(dtype)
+    return t.cuda()
+
+
+def host(t):
+    """cuda tensor -> numpy; 16-bit floats come back as uint16 bit patterns, e4m3 as uint8."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype in (torch.bfloat16, torch.float16):
+        return t.view(torch.int16).numpy().view(np.uint16)
+    if t.dtype == torch.float8_e4m3fn:
+        return t.view(torch.uint8).numpy()
+    return t.numpy()
+
+
+def bf16_normal(shape, seed, scale=1.0):
+    return zo.f32_to_bf16((rng(seed).standard_normal(shape) * scale).astype(np.float32))
+
+
+def distinct_topk(T, E, K, seed, zipf=None):
+    """K distinct experts per token; uniform, or Zipf(s)-skewed popularity over a fixed random permutation."""
+    g = rng(seed)
+    if zipf is None:
+        return np.stack([g.permutation(E)[:K] for _ in range(T)]).astype(np.int64)
+    p = 1.0 / np.arange(1, E + 1) ** zipf
+    p = p[g.permutation(E)]
+    p /= p.sum()
+    return np.stack([g.choice(E, size=K, replace=False, p=p) for _ in range(T)]).astype(np.int64)
+
+
+def calc_diff(x, y):
+    """Reference metric, app/zbal/test/python/deepep/utils.py:129-133."""
+    x = x.astype(np.float64) + 1
+    y = y.astype(np.float64) + 1
+    return 1 - 2 * (x * y).sum() / (x * x + y * y).sum()
+
+
+def max_rel_err(got, want):
+    """max |got - want| relative to the largest reference magnitude."""
+    got = got.astype(np.float64)
+    want = want.astype(np.float64)
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
