@@ -1,0 +1,241 @@
+#!/usr/bin/env python3
+"""Benchmark of the MoE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+One step = one pass of the layer over one batch already resident in HBM:
+softmax top-k router -> zbal_fused_deep_moe (permute + fp8 quantise, grouped
+GEMM 1 with SwiGLU + requantise, grouped GEMM 2, weighted combine), all through
+the zbal C ABI. The workload is the DeepSeek-V3-style prefill share: 4096
+tokens x hidden 7168, 32 local experts, top-8 over uniform-random logits, fp8
+e4m3 with 1x128 activation and 128x128 weight scales, intermediate 2048.
+Synthetic data, random weights.
+
+Prints ONE JSON line. `value` is tokens/s of the whole step. `roofline`
+prices the dominant kernel (grouped GEMM 1) from its algorithmic FLOPs and
+its average duration measured with HIP events in a second loop that issues
+the same stages one by one through the inner kernel ABI. `cpu_baseline` is
+the CPU oracle (a scalar C++ restatement, OpenMP over rows) timed on the
+host on a bounded sample of the same batch; the same sample is used to check
+the GPU result.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA
+PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--tokens", type=int, default=4096, help="development only; the reported workload is 4096")
+    ap.add_argument("--cpu-sample-tokens", type=int, default=128)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    return ap.parse_args()
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        sys.stderr.write("bench.py: this build measures one GPU's share of the path; runs with --gpus > 1 are not "
+                         "part of it (no collectives, no sharding). Use --gpus 1.\n")
+        sys.exit(2)
+
+    import numpy as np
+    import torch
+    from memfabric_hybrid_amd import capi
+    from memfabric_hybrid_amd.buffer import Buffer
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    dev = torch.device("cuda", 0)
+    buf = Buffer()
+    lib = buf.lib
+
+    T, H, E, K, I = args.tokens, 7168, 32, 8, 2048
+    N1 = 2 * I
+    rows = T * K
+    torch.manual_seed(0)
+    x = torch.randn((T, H), device=dev, dtype=torch.float32).to(torch.bfloat16)
+    logits = torch.rand((T, E), device=dev, dtype=torch.float32)
+
+    def fp8_weight(k, n):
+        w = torch.empty((E, k, n), device=dev, dtype=torch.float8_e4m3fn)
+        for e in range(E):
+            w[e] = (torch.randn((k, n), device=dev, dtype=torch.float32) * 100.0).clamp_(-448, 448).to(torch.float8_e4m3fn)
+        return w
+
+    w1_logical = fp8_weight(H, N1)                       # [E, K, N] as the operator API describes them
+    w2_logical = fp8_weight(I, H)
+    w1 = buf.prepack_weight(w1_logical)                  # [E, N, K] K-contiguous
+    w2 = buf.prepack_weight(w2_logical)
+    s1 = (torch.rand((E, H // 128, N1 // 128), device=dev) + 0.5) * (1.0 / (100.0 * H ** 0.5))
+    s2 = (torch.rand((E, I // 128, H // 128), device=dev) + 0.5) * (1.0 / (100.0 * I ** 0.5))
+    torch.cuda.synchronize()
+
+    qmode = capi.QUANT_FP8_B128
+    ws = torch.empty(buf.fused_workspace_bytes(T, H, K, E, N1, qmode), dtype=torch.uint8, device=dev)
+    out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
+    topk_idx = torch.empty((T, K), dtype=torch.int64, device=dev)
+    topk_w = torch.empty((T, K), dtype=torch.float32, device=dev)
+    ids32 = torch.empty((T, K), dtype=torch.int32, device=dev)
+    nums = torch.empty(E, dtype=torch.int64, device=dev)
+
+    ti = capi.tensor_info
+    null = capi.TensorInfo()
+    d = dict(x=ti(x), logits=ti(logits), idx=ti(topk_idx), w=ti(topk_w), ids=ti(ids32),
+             w1=ti(w1, dtype=capi.DT_FP8_E4M3, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s1=ti(s1),
+             w2=ti(w2, dtype=capi.DT_FP8_E4M3, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s2=ti(s2),
+             out=ti(out), nums=ti(nums), ws=ti(ws))
+    r = ctypes.byref
+    st = capi.stream_ptr()
+
+    def step():
+        capi.check("route", lib.zbal_moe_topk_route(r(d["logits"]), K, r(d["idx"]), r(d["w"]), buf.comm, st, 0))
+        ids32.copy_(topk_idx)                            # the adaptor's int64 -> int32 cast (zbal_deepep.cpp:316)
+        capi.check("fused", lib.zbal_fused_deep_moe(
+            r(d["x"]), r(d["ids"]), r(d["w1"]), r(d["s1"]), r(d["w2"]), r(d["s2"]), r(d["w"]), r(null), r(null), r(null),
+            r(null), r(null), r(null), r(null), r(d["out"]), r(null), r(d["nums"]), r(d["ws"]), E, qmode, 0, N1, 0, 0,
+            buf.comm, st, 0))
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(args.steps):
+        step()
+    e1.record()
+    torch.cuda.synchronize()
+    ms_per_step = e0.elapsed_time(e1) / args.steps
+    out_fused = out.clone()
+
+    # ---- the same stages one by one through the inner kernel ABI, with events between them -----------------
+    off = {k: int(v) for k, v in plan_workspace(lib, T, H, K, E, N1, qmode).items()}
+    base = ws.data_ptr()
+    q1, xs, eidx, row_off, scratch, q2, sc2, y = (base + off[k] for k in
+                                                  ("q1", "xs", "expand_idx", "row_off", "layout_scratch", "q2", "scale2", "y"))
+    names = ["route", "permute_quant", "gmm1_swiglu_quant", "gmm2_dequant", "combine"]
+
+    def staged(evs):
+        evs[0].record()
+        capi.check("route", lib.zbalhip_topk_route(logits.data_ptr(), T, E, K, topk_idx.data_ptr(), topk_w.data_ptr(), st))
+        ids32.copy_(topk_idx)
+        evs[1].record()
+        capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, T, H, K, E, 2,
+                                                              q1, xs, eidx, nums.data_ptr(), row_off, scratch, 50, st))
+        evs[2].record()
+        capi.check("gmm1", lib.zbalhip_gmm1_swiglu_quant(q1, xs, w1.data_ptr(), s1.data_ptr(), row_off, E, rows, H, N1, 2,
+                                                         q2, sc2, None, st))
+        evs[3].record()
+        capi.check("gmm2", lib.zbalhip_gmm2_dequant(q2, sc2, w2.data_ptr(), s2.data_ptr(), capi.DT_FP32, row_off, E, rows, I,
+                                                    H, 2, capi.DT_BF16, y, st))
+        evs[4].record()
+        capi.check("combine", lib.zbalhip_combine(y, capi.DT_BF16, row_off, 0, topk_w.data_ptr(), ids32.data_ptr(), eidx, T, H,
+                                                  K, E, out.data_ptr(), st))
+        evs[5].record()
+
+    all_evs = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]
+    for _ in range(max(1, args.warmup // 2)):
+        staged([torch.cuda.Event(enable_timing=True) for _ in range(6)])
+    torch.cuda.synchronize()
+    for evs in all_evs:
+        staged(evs)
+    torch.cuda.synchronize()
+    stage_ms = {n: sum(evs[i].elapsed_time(evs[i + 1]) for evs in all_evs) / args.steps for i, n in enumerate(names)}
+    assert torch.equal(out, out_fused), "staged and fused paths disagree"
+
+    flops1 = 2.0 * rows * H * N1
+    flops2 = 2.0 * rows * I * H
+    bytes_permute = T * H * 2 + rows * (H + H // 128 * 4)
+    bytes_combine = rows * H * 2 + T * H * 2
+    t1 = stage_ms["gmm1_swiglu_quant"] * 1e-3
+    roofline = {"kernel": "grouped_gemm_kernel<fp8, gmm1>", "bound": "mfma", "achieved": flops1 / t1 / 1e12,
+                "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS, "traffic": None}
+    stages = {
+        "ms": {k: round(v, 4) for k, v in stage_ms.items()},
+        "gmm2_tflops": flops2 / (stage_ms["gmm2_dequant"] * 1e-3) / 1e12,
+        "permute_quant_gbs": bytes_permute / (stage_ms["permute_quant"] * 1e-3) / 1e9,
+        "combine_gbs": bytes_combine / (stage_ms["combine"] * 1e-3) / 1e9,
+        "permute_quant_frac_hbm": bytes_permute / (stage_ms["permute_quant"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+        "combine_frac_hbm": bytes_combine / (stage_ms["combine"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
+    }
+
+    # ---- CPU baseline on a bounded sample, which also checks the GPU result -------------------------------------
+    cpu = None
+    parity = None
+    if not args.no_cpu:
+        from oracle import oracle as zo
+        ts = min(args.cpu_sample_tokens, T)
+        xs_np = x[:ts].view(torch.int16).cpu().numpy().view(np.uint16)
+        ids_np = ids32[:ts].cpu().numpy()
+        w_np = topk_w[:ts].cpu().numpy()
+        w1_np = w1_logical.view(torch.uint8).cpu().numpy()
+        w2_np = w2_logical.view(torch.uint8).cpu().numpy()
+        s1_np, s2_np = s1.cpu().numpy(), s2.cpu().numpy()
+        t0 = time.perf_counter()
+        ref, _ = zo.fused_moe(xs_np, zo.DT_BF16, ids_np, w_np, w1_np, s1_np, w2_np, s2_np, E, 2)
+        secs = time.perf_counter() - t0
+        got = zo.bf16_to_f32(out_fused[:ts].view(torch.int16).cpu().numpy().view(np.uint16))
+        want = zo.bf16_to_f32(ref)
+        err = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+        parity = {"tokens": ts, "max_rel_err": err, "tolerance": 2e-2, "ok": bool(err < 2e-2)}
+        cpu = {"value": ts / secs, "unit": "tokens/s", "cores": zo.num_threads(), "kind": "port",
+               "sample": "first %d tokens of the same batch (%d expert rows, all %d experts' weights), %.1f s" %
+                         (ts, ts * K, E, secs)}
+
+    line = {
+        "metric": "MoE layer tokens/s at 1 GPU", "value": T / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3", "data": "synthetic",
+        "config": {"workload": "DeepSeek-V3-style prefill share (BASELINE configs[1])", "tokens": T, "hidden": H,
+                   "experts": E, "topk": K, "intermediate": I, "quant": "fp8 e4m3, act 1x128, weight 128x128",
+                   "parallelism": "1 GPU"},
+        "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "parity": parity,
+    }
+    print(json.dumps(line))
+    buf.close()
+
+
+def plan_workspace(lib, T, H, K, E, N1, qmode):
+    """Offsets of the fused operator's workspace regions; mirrors PlanFusedWorkspace in the host layer
+    (csrc/host/zbal_gpu_communicator.cpp) and is cross-checked against the size the library reports."""
+    rows = max(T * K, 1)
+    I = N1 // 2
+    fp8 = qmode == 2
+    off = {}
+    cur = 0
+
+    def take(name, nbytes):
+        nonlocal cur
+        off[name] = cur
+        cur = (cur + nbytes + 255) & ~255
+
+    take("q1", rows * H)
+    take("xs", rows * (H // 128 if fp8 else 1) * 4)
+    take("expand_idx", rows * 4)
+    take("counts", E * 8)
+    take("row_off", (E + 1) * 4)
+    take("layout_scratch", 50 * E * 4)
+    take("q2", rows * I)
+    take("scale2", rows * ((I + 127) // 128 if fp8 else 1) * 4)
+    if not fp8:
+        take("sgl", rows * (I + 1) * 4)
+    take("y", rows * H * 2)
+    assert cur == lib.zbal_fused_deep_moe_workspace_size(T, H, K, E, N1, qmode), "workspace plan out of sync"
+    return off
+
+
+if __name__ == "__main__":
+    main()

@@ -127,6 +127,9 @@ def load():
     if not os.path.exists(LIB_PATH):
         raise RuntimeError("libzbal.so is missing (%s): build it with `python -m memfabric_hybrid_amd.build`; "
                            "there is no fallback implementation" % LIB_PATH)
+    # Device memory comes from torch, so the library must bind to the HIP runtime torch ships: import torch
+    # first so that its libamdhip64 is the one already resident when libzbal.so resolves its dependency.
+    import torch  # noqa: F401
     lib = ctypes.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)

@@ -104,7 +104,7 @@ public:
     static size_t ElemSize(zbal_datatype_t dt)
     {
         switch (dt) {
-            case ZBAL_DATA_TYPE_INT8: case ZBAL_DATA_TYPE_UINT8: return 1;
+            case ZBAL_DATA_TYPE_INT8: case ZBAL_DATA_TYPE_UINT8: case ZBAL_DATA_TYPE_FP8_E4M3: case ZBAL_DATA_TYPE_INT4X2: return 1;
             case ZBAL_DATA_TYPE_INT16: case ZBAL_DATA_TYPE_UINT16: case ZBAL_DATA_TYPE_FP16: case ZBAL_DATA_TYPE_BFP16: return 2;
             case ZBAL_DATA_TYPE_INT32: case ZBAL_DATA_TYPE_UINT32: case ZBAL_DATA_TYPE_FP32: return 4;
             case ZBAL_DATA_TYPE_INT64: case ZBAL_DATA_TYPE_UINT64: case ZBAL_DATA_TYPE_FP64: return 8;

@@ -645,6 +645,7 @@ ZO_API void zo_gmm1_swiglu_quant_fp8(const uint8_t *a, const float *sa, const ui
     std::vector<float> wf(size_t(K) * N1);
     for (int64_t g = 0; g < E; ++g) {
         if (counts[g] == 0) continue;
+#pragma omp parallel for schedule(static)
         for (int64_t i = 0; i < K * N1; ++i) wf[i] = e4m3_to_f32(w1[g * K * N1 + i]);
 #pragma omp parallel for schedule(static)
         for (int64_t m = off[g]; m < off[g + 1]; ++m) {
@@ -670,6 +671,7 @@ ZO_API void zo_gmm2_fp8(const uint8_t *a, const float *sa, const uint8_t *w2, co
     std::vector<float> wf(size_t(K) * N);
     for (int64_t g = 0; g < E; ++g) {
         if (counts[g] == 0) continue;
+#pragma omp parallel for schedule(static)
         for (int64_t i = 0; i < K * N; ++i) wf[i] = e4m3_to_f32(w2[g * K * N + i]);
 #pragma omp parallel for schedule(static)
         for (int64_t m = off[g]; m < off[g + 1]; ++m) {

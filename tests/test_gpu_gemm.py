@@ -167,9 +167,9 @@ def fused_inputs(T, H, K, E, I, mode, seed, zipf=None):
         s2 = zo.f32_to_bf16(rng(seed + 6).uniform(0.0015, 0.0045, (E, H)).astype(np.float32))
     elif mode == 2:
         w1 = zo.f32_to_e4m3(rng(seed + 3).standard_normal((E, H, 2 * I)).astype(np.float32) * 100)
-        s1 = rng(seed + 4).uniform(0.5, 1.5, (E, H // 128, 2 * I // 128)).astype(np.float32) * 2e-4 / np.sqrt(H / 256)
+        s1 = (rng(seed + 4).uniform(0.5, 1.5, (E, H // 128, 2 * I // 128)) * 2e-4 / np.sqrt(H / 256)).astype(np.float32)
         w2 = zo.f32_to_e4m3(rng(seed + 5).standard_normal((E, I, H)).astype(np.float32) * 100)
-        s2 = rng(seed + 6).uniform(0.5, 1.5, (E, I // 128, H // 128)).astype(np.float32) * 2e-4
+        s2 = (rng(seed + 6).uniform(0.5, 1.5, (E, I // 128, H // 128)) * 2e-4).astype(np.float32)
     else:
         w1 = rng(seed + 3).integers(-8, 8, (E, H, 2 * I)).astype(np.int8)
         s1 = zo.f32_to_fp16(rng(seed + 4).uniform(0.003, 0.009, (E, H // 128, 2 * I)).astype(np.float32))
