@@ -66,6 +66,7 @@ struct TileCoord {
 };
 
 /* wave-uniform search of the logical tile this workgroup owns; false = nothing to do */
+template <int TILE_M>
 __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ row_off, int experts, int n_tiles,
                                             TileCoord &tc)
 {
@@ -74,7 +75,7 @@ __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ row_off,
     for (int base = 0; base < experts; base += 64) {
         const int e = base + lane;
         int t = 0;
-        if (e < experts) t = ((row_off[e + 1] - row_off[e] + BM - 1) / BM) * n_tiles;
+        if (e < experts) t = ((row_off[e + 1] - row_off[e] + TILE_M - 1) / TILE_M) * n_tiles;
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
         total += t;
@@ -89,7 +90,7 @@ __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ row_off,
     for (int base = 0; base < experts; base += 64) {
         const int e = base + lane;
         int mt = 0;
-        if (e < experts) mt = (row_off[e + 1] - row_off[e] + BM - 1) / BM;
+        if (e < experts) mt = (row_off[e + 1] - row_off[e] + TILE_M - 1) / TILE_M;
         const int t = mt * n_tiles;
         int incl = t;
 #pragma unroll
@@ -120,8 +121,6 @@ __device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ row_off,
     return true;
 }
 
-typedef float f32x4_t __attribute__((ext_vector_type(4)));
-
 __device__ __forceinline__ f32x4 mfma_fp8_16x16x128(const i32x8 &wfrag, const i32x8 &afrag)
 {
     const f32x4 zero = {0.0f, 0.0f, 0.0f, 0.0f};
@@ -133,6 +132,133 @@ __device__ __forceinline__ f32x4 mfma_fp8_16x16x128(const i32x8 &wfrag, const i3
 __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float d)
 {
     return zb_cvt_pk_e4m3(a, b) | (zb_cvt_pk_e4m3(c, d) << 16);
+}
+
+/*
+ * Shared epilogue. The calling wave holds, for sub-tile (mt, nt), output channels 4*(lane/16)+i of token
+ * row wm*64 + mt*16 + lane%16. `lds_rowmax` is [2][tile_rows] floats of scratch for the row maxima of the
+ * two channel halves (GMM1 only).
+ */
+template <int MODE, bool GMM1, int OUT_DT>
+__device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &tc, f32x4 (&accf)[4][8],
+                                         i32x4 (&acci)[4][8], int row_begin, int row_end, int wm, int wn, int lane,
+                                         float *lds_rowmax, int tile_rows)
+{
+    const int frag_row = lane & 15;
+    const int I = p.N / 2;
+    const int sub_n = (lane >> 4) * 4;
+    if constexpr (!GMM1) {
+        uint16_t *y = (uint16_t *)p.out;
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
+            if (row >= row_end) continue;
+            float xs = 1.0f;
+            if (MODE != MODE_FP8) xs = p.a_scale[row];
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) {
+                const int n = tc.n_tile * BN + wn * 128 + nt * 16 + sub_n;
+                float d[4];
+                if constexpr (MODE == MODE_W8A8) {
+                    float ws[4];
+                    if (p.wscale_is_bf16) {
+                        const u32x2 v = *reinterpret_cast<const u32x2 *>((const uint16_t *)p.wscale + (int64_t)tc.expert * p.N + n);
+                        ws[0] = zb_bf16_to_f32(v[0] & 0xffffu); ws[1] = zb_bf16_to_f32(v[0] >> 16);
+                        ws[2] = zb_bf16_to_f32(v[1] & 0xffffu); ws[3] = zb_bf16_to_f32(v[1] >> 16);
+                    } else {
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>((const float *)p.wscale + (int64_t)tc.expert * p.N + n);
+                        ws[0] = v[0]; ws[1] = v[1]; ws[2] = v[2]; ws[3] = v[3];
+                    }
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) d[i] = ((float)acci[mt][nt][i] * ws[i]) * xs;
+                } else if constexpr (MODE == MODE_FP8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i];
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i] * xs;
+                }
+                u32x2 o;
+                o[0] = zb_f32_to_half<OUT_DT>(d[0]) | (zb_f32_to_half<OUT_DT>(d[1]) << 16);
+                o[1] = zb_f32_to_half<OUT_DT>(d[2]) | (zb_f32_to_half<OUT_DT>(d[3]) << 16);
+                *reinterpret_cast<u32x2 *>(y + (int64_t)row * p.N + n) = o;
+            }
+        }
+    } else {
+        /* SwiGLU on gate sub-tile nt and up sub-tile nt+4: columns j = n_tile*128 + wn*64 + nt*16 + sub_n + i */
+        float sg[4][4][4];
+        float rmax[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
+            int lrow = row;
+            if (lrow > p.max_rows - 1) lrow = p.max_rows - 1;
+            float xs = 1.0f;
+            if (MODE != MODE_FP8) xs = p.a_scale[lrow];
+            rmax[mt] = 0.0f;
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+                const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                float g[4], u[4];
+                if constexpr (MODE == MODE_W8A8) {
+                    const float *wsb = (const float *)p.wscale + (int64_t)tc.expert * p.N;
+                    const f32x4 wg = *reinterpret_cast<const f32x4 *>(wsb + j);
+                    const f32x4 wu = *reinterpret_cast<const f32x4 *>(wsb + I + j);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        g[i] = ((float)acci[mt][nt][i] * wg[i]) * xs;
+                        u[i] = ((float)acci[mt][nt + 4][i] * wu[i]) * xs;
+                    }
+                } else if constexpr (MODE == MODE_FP8) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { g[i] = accf[mt][nt][i]; u[i] = accf[mt][nt + 4][i]; }
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) { g[i] = accf[mt][nt][i] * xs; u[i] = accf[mt][nt + 4][i] * xs; }
+                }
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float left = g[i] / (1.0f + zb_expf(-g[i]));
+                    const float s = left * u[i];
+                    sg[mt][nt][i] = s;
+                    rmax[mt] = fmaxf(rmax[mt], fabsf(s));
+                }
+            }
+            /* the four lane groups (lane/16) hold different columns of the same row */
+            rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 16, 64));
+            rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 32, 64));
+            if (lane < 16) lds_rowmax[wn * tile_rows + wm * 64 + mt * 16 + lane] = rmax[mt];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) {
+            const int lr = wm * 64 + mt * 16 + frag_row;
+            const int row = row_begin + lr;
+            const float amax_tile = fmaxf(lds_rowmax[lr], lds_rowmax[tile_rows + lr]);
+            if (row >= row_end) continue;
+            if constexpr (MODE == MODE_FP8) {
+                const float amax = fmaxf(amax_tile, 1e-4f);
+                const float mult = 448.0f / amax;
+                uint8_t *q2 = (uint8_t *)p.out;
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                    const uint32_t v = pack4_e4m3(sg[mt][nt][0] * mult, sg[mt][nt][1] * mult, sg[mt][nt][2] * mult,
+                                                  sg[mt][nt][3] * mult);
+                    *reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I + j) = v;
+                }
+                if (wn == 0 && lane < 16) p.out_scale[(int64_t)row * (I / 128) + tc.n_tile] = amax * (1.0f / 448.0f);
+            } else {
+#pragma unroll
+                for (int nt = 0; nt < 4; ++nt) {
+                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                    const f32x4 v = f32x4{sg[mt][nt][0], sg[mt][nt][1], sg[mt][nt][2], sg[mt][nt][3]};
+                    *reinterpret_cast<f32x4 *>(p.sgl_ws + (int64_t)row * I + j) = v;
+                }
+                if (wn == 0 && lane < 16) atomicMax(&p.rowmax[row], __float_as_uint(amax_tile));
+            }
+        }
+    }
 }
 
 template <int MODE, bool GMM1, int OUT_DT>
@@ -147,7 +273,7 @@ grouped_gemm_kernel(GemmParams p)
 
     const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
     TileCoord tc;
-    if (!locate_tile(p.row_off, p.experts, n_tiles, tc)) return;
+    if (!locate_tile<BM>(p.row_off, p.experts, n_tiles, tc)) return;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -344,121 +470,201 @@ grouped_gemm_kernel(GemmParams p)
         }
     }
 
-    /* ---- epilogue ------------------------------------------------------------------------- */
-    /* lane owns token row m = row_begin + wm*64 + mt*16 + lane%16 and channels 4*(lane/16)+i of each 16-wide sub-tile */
-    const int sub_n = (lane >> 4) * 4;
-    if constexpr (!GMM1) {
-        uint16_t *y = (uint16_t *)p.out;
+    epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, row_begin, row_end, wm, wn, lane, &lds_rowmax[0][0], BM);
+}
+
+/* ------------------------------------------------------------------------------------------------------
+ * Large-tile kernel for the 8-bit modes (W8A8, fp8): 256 token rows x 256 channels x 128 K-bytes per
+ * workgroup, eight waves in a 4 x 2 grid (same 64 x 128 wave tile as above), one workgroup per CU.
+ *
+ * K slabs go from HBM to LDS without passing through registers: every wave issues
+ * global_load_lds_dwordx4, which deposits the 64 lanes' 16-byte chunks in 1 KiB of consecutive LDS
+ * (lane l at +16*l). A block of 1 KiB holds 8 tile rows of 128 bytes; which global chunk a lane fetches is
+ * free, so the chunk stored in slot s of row r is logical chunk s ^ ((r >> 1) & 7). With that XOR the 16
+ * rows a fragment read touches (same logical chunk, 128-byte pitch) fall into 16 distinct groups of four
+ * banks, which plain row-major storage would collapse onto two. Two stages of 64 KiB alternate: the slab
+ * for step k+1 is in flight while step k is multiplied, with one barrier per step.
+ * ------------------------------------------------------------------------------------------------------ */
+constexpr int DM = 256;
+constexpr int DTHREADS = 512;
+constexpr int D_A_BYTES = DM * BKB;
+constexpr int D_STAGE_BYTES = (DM + BN) * BKB;
+constexpr int D_MAX_KB = 256;                 /* K up to 32768 */
+constexpr int D_LDS_BYTES = 2 * D_STAGE_BYTES + 2 * DM * 4 + 2 * DM * 4 + 2 * D_MAX_KB * 4;
+
+__device__ __forceinline__ void dma16(const uint8_t *g, uint8_t *lds_wave_base)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                     (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
+}
+
+__device__ __forceinline__ void dma4(const float *g, float *lds_wave_base)
+{
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
+                                     (__attribute__((address_space(3))) void *)lds_wave_base, 4, 0, 0);
+}
+
+template <int MODE, bool GMM1, int OUT_DT>
+__global__ void __launch_bounds__(DTHREADS, 2)
+grouped_gemm_dma_kernel(GemmParams p)
+{
+    static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8, "int4 weights need the register-staged kernel");
+    extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
+    float *lds_sa = reinterpret_cast<float *>(smem + 2 * D_STAGE_BYTES);   /* [2][DM] */
+    float *lds_rowmax = lds_sa + 2 * DM;                                   /* [2][DM] */
+    float *lds_sw = lds_rowmax + 2 * DM;                                   /* [2][D_MAX_KB] fp8 weight block scales */
+
+    const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
+    TileCoord tc;
+    if (!locate_tile<DM>(p.row_off, p.experts, n_tiles, tc)) return;
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wm = wave >> 1, wn = wave & 1;
+    const int row_begin = p.row_off[tc.expert] + tc.m_tile * DM;
+    const int row_end = p.row_off[tc.expert + 1];
+    const int K = p.K;
+    const int KB = K / 128;
+    const int I = p.N / 2;
+
+    /* DMA sources: this wave fills blocks wave + 8*i (i = 0..3) of the A tile and of the W tile */
+    const uint8_t *a_src[4];
+    const uint8_t *w_src[4];
+    {
+        const int rr = lane >> 3, slot = lane & 7;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = 8 * (wave + 8 * i) + rr;
+            const int c = slot ^ ((r >> 1) & 7);
+            int gr = row_begin + r;
+            if (gr > p.max_rows - 1) gr = p.max_rows - 1;
+            a_src[i] = p.a + (int64_t)gr * K + c * 16;
+            int wrow;
+            if (GMM1) wrow = (r < 128) ? tc.n_tile * 128 + r : I + tc.n_tile * 128 + (r - 128);
+            else wrow = tc.n_tile * BN + r;
+            w_src[i] = p.w + ((int64_t)tc.expert * p.N + wrow) * K + c * 16;
+        }
+    }
+    const float *sa_src = nullptr;
+    if (MODE == MODE_FP8 && wave < 4) {
+        int gr = row_begin + wave * 64 + lane;
+        if (gr > p.max_rows - 1) gr = p.max_rows - 1;
+        sa_src = p.a_scale + (int64_t)gr * KB;
+    }
+    if (MODE == MODE_FP8) {
+        /* the two weight block scales of every K slab of this tile, fetched once (visible after the first barrier) */
+        const int sw_stride = p.N / 128;
+        const float *base = (const float *)p.wscale + (int64_t)tc.expert * KB * sw_stride;
+        const int c0 = GMM1 ? tc.n_tile : tc.n_tile * 2, c1 = GMM1 ? I / 128 + tc.n_tile : tc.n_tile * 2 + 1;
+        for (int kb = tid; kb < KB; kb += DTHREADS) {
+            lds_sw[kb] = base[(int64_t)kb * sw_stride + c0];
+            lds_sw[D_MAX_KB + kb] = base[(int64_t)kb * sw_stride + c1];
+        }
+    }
+
+    auto issue = [&](int kb, int stage) {
+        uint8_t *sb = smem + stage * D_STAGE_BYTES;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(a_src[i] + (int64_t)kb * BKB, sb + (wave + 8 * i) * 1024);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) dma16(w_src[i] + (int64_t)kb * BKB, sb + D_A_BYTES + (wave + 8 * i) * 1024);
+        if (MODE == MODE_FP8 && wave < 4) dma4(sa_src + kb, lds_sa + stage * DM + wave * 64);
+    };
+
+    f32x4 accf[4][8];
+    i32x4 acci[4][8];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 8; ++nt) {
+            accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            acci[mt][nt] = i32x4{0, 0, 0, 0};
+        }
+
+    /* fragment reads: row lane%16 of a 16-row sub-tile, logical chunks 2*(lane/16) and 2*(lane/16)+1 */
+    const int frag_row = lane & 15;
+    const int key = (lane >> 1) & 7, g2 = (lane >> 4) * 2;
+    const int off_lo = frag_row * BKB + ((g2 ^ key) * 16), off_hi = frag_row * BKB + (((g2 + 1) ^ key) * 16);
+    int w_sub[8];
+#pragma unroll
+    for (int nt = 0; nt < 8; ++nt) {
+        int r;
+        if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
+        else r = wn * 128 + nt * 16;
+        w_sub[nt] = D_A_BYTES + r * BKB;
+    }
+
+    issue(0, 0);
+    for (int kb = 0; kb < KB; ++kb) {
+        const int stage = kb & 1;
+        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's DMA for slab kb has landed */
+        __syncthreads();                    /* ... and everybody else's; stage^1 is free again */
+        if (kb + 1 < KB) issue(kb + 1, stage ^ 1);
+        const uint8_t *sb = smem + stage * D_STAGE_BYTES;
+
+        auto load_w = [&](int nt) -> i32x8 {
+            const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
+            const u32x4 hi = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_hi);
+            return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        };
+        i32x8 af[4];
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
-            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
-            if (row >= row_end) continue;
-            float xs = 1.0f;
-            if (MODE != MODE_FP8) xs = p.a_scale[row];
+            const uint8_t *ab = sb + (wm * 64 + mt * 16) * BKB;
+            const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
+            const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
+            af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+        }
+
+        if constexpr (MODE == MODE_FP8) {
+            /*
+             * Software pipeline over the 32 (channel sub-tile, row sub-tile) pairs: the MFMA of pair p+1 is issued
+             * before the four scale-and-accumulate FMAs of pair p, so the vector ALU works under the matrix unit.
+             */
+            const float sw0 = lds_sw[kb], sw1 = lds_sw[D_MAX_KB + kb];
+            float s0[4], s1[4];
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt) {
+                const float sa = lds_sa[stage * DM + wm * 64 + mt * 16 + frag_row];
+                s0[mt] = sa * sw0;
+                s1[mt] = sa * sw1;
+            }
+            i32x8 wf = load_w(0);
+            f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
 #pragma unroll
             for (int nt = 0; nt < 8; ++nt) {
-                const int n = tc.n_tile * BN + wn * 128 + nt * 16 + sub_n;
-                float d[4];
-                if constexpr (MODE == MODE_W8A8) {
-                    float ws[4];
-                    if (p.wscale_is_bf16) {
-                        const u32x2 v = *reinterpret_cast<const u32x2 *>((const uint16_t *)p.wscale + (int64_t)tc.expert * p.N + n);
-                        ws[0] = zb_bf16_to_f32(v[0] & 0xffffu); ws[1] = zb_bf16_to_f32(v[0] >> 16);
-                        ws[2] = zb_bf16_to_f32(v[1] & 0xffffu); ws[3] = zb_bf16_to_f32(v[1] >> 16);
-                    } else {
-                        const f32x4 v = *reinterpret_cast<const f32x4 *>((const float *)p.wscale + (int64_t)tc.expert * p.N + n);
-                        ws[0] = v[0]; ws[1] = v[1]; ws[2] = v[2]; ws[3] = v[3];
-                    }
+                i32x8 wf_n = wf;
+                if (nt + 1 < 8) wf_n = load_w(nt + 1);
+                const bool second = GMM1 ? (nt >= 4) : (wn == 1);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) d[i] = ((float)acci[mt][nt][i] * ws[i]) * xs;
-                } else if constexpr (MODE == MODE_FP8) {
+                for (int mt = 0; mt < 4; ++mt) {
+                    f32x4 nxt = part;
+                    if (mt < 3) nxt = mfma_fp8_16x16x128(wf, af[mt + 1]);
+                    else if (nt + 1 < 8) nxt = mfma_fp8_16x16x128(wf_n, af[0]);
+                    const float sc = second ? s1[mt] : s0[mt];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i];
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i] * xs;
+                    for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
+                    part = nxt;
                 }
-                u32x2 o;
-                o[0] = zb_f32_to_half<OUT_DT>(d[0]) | (zb_f32_to_half<OUT_DT>(d[1]) << 16);
-                o[1] = zb_f32_to_half<OUT_DT>(d[2]) | (zb_f32_to_half<OUT_DT>(d[3]) << 16);
-                *reinterpret_cast<u32x2 *>(y + (int64_t)row * p.N + n) = o;
+                wf = wf_n;
             }
-        }
-    } else {
-        /* SwiGLU on gate sub-tile nt and up sub-tile nt+4: columns j = n_tile*128 + wn*64 + nt*16 + sub_n + i */
-        float sg[4][4][4];
-        float rmax[4];
+        } else {
+            /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
-            int lrow = row;
-            if (lrow > p.max_rows - 1) lrow = p.max_rows - 1;
-            float xs = 1.0f;
-            if (MODE != MODE_FP8) xs = p.a_scale[lrow];
-            rmax[mt] = 0.0f;
+            for (int nt = 0; nt < 8; ++nt) {
+                const i32x8 wf = load_w(nt);
+                const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
 #pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-                const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
-                float g[4], u[4];
-                if constexpr (MODE == MODE_W8A8) {
-                    const float *wsb = (const float *)p.wscale + (int64_t)tc.expert * p.N;
-                    const f32x4 wg = *reinterpret_cast<const f32x4 *>(wsb + j);
-                    const f32x4 wu = *reinterpret_cast<const f32x4 *>(wsb + I + j);
+                for (int mt = 0; mt < 4; ++mt)
+                    acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                        wf0, i32x4{af[mt][0], af[mt][1], af[mt][2], af[mt][3]}, acci[mt][nt], 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        g[i] = ((float)acci[mt][nt][i] * wg[i]) * xs;
-                        u[i] = ((float)acci[mt][nt + 4][i] * wu[i]) * xs;
-                    }
-                } else if constexpr (MODE == MODE_FP8) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { g[i] = accf[mt][nt][i]; u[i] = accf[mt][nt + 4][i]; }
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) { g[i] = accf[mt][nt][i] * xs; u[i] = accf[mt][nt + 4][i] * xs; }
-                }
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float left = g[i] / (1.0f + zb_expf(-g[i]));
-                    const float s = left * u[i];
-                    sg[mt][nt][i] = s;
-                    rmax[mt] = fmaxf(rmax[mt], fabsf(s));
-                }
-            }
-            /* the four lane groups (lane/16) hold different columns of the same row */
-            rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 16, 64));
-            rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 32, 64));
-            if (lane < 16) lds_rowmax[wn][wm * 64 + mt * 16 + lane] = rmax[mt];
-        }
-        __syncthreads();
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-            const int lr = wm * 64 + mt * 16 + frag_row;
-            const int row = row_begin + lr;
-            const float amax_tile = fmaxf(lds_rowmax[0][lr], lds_rowmax[1][lr]);
-            if (row >= row_end) continue;
-            if constexpr (MODE == MODE_FP8) {
-                const float amax = fmaxf(amax_tile, 1e-4f);
-                const float mult = 448.0f / amax;
-                uint8_t *q2 = (uint8_t *)p.out;
-#pragma unroll
-                for (int nt = 0; nt < 4; ++nt) {
-                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
-                    const uint32_t v = pack4_e4m3(sg[mt][nt][0] * mult, sg[mt][nt][1] * mult, sg[mt][nt][2] * mult,
-                                                  sg[mt][nt][3] * mult);
-                    *reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I + j) = v;
-                }
-                if (wn == 0 && lane < 16) p.out_scale[(int64_t)row * (I / 128) + tc.n_tile] = amax * (1.0f / 448.0f);
-            } else {
-#pragma unroll
-                for (int nt = 0; nt < 4; ++nt) {
-                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
-                    const f32x4 v = f32x4{sg[mt][nt][0], sg[mt][nt][1], sg[mt][nt][2], sg[mt][nt][3]};
-                    *reinterpret_cast<f32x4 *>(p.sgl_ws + (int64_t)row * I + j) = v;
-                }
-                if (wn == 0 && lane < 16) atomicMax(&p.rowmax[row], __float_as_uint(amax_tile));
+                for (int mt = 0; mt < 4; ++mt)
+                    acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                        wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
             }
         }
     }
+    epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, row_begin, row_end, wm, wn, lane, lds_rowmax, DM);
 }
 
 /* second pass of the int8 GMM1 epilogue: whole-row requantisation from the fp32 SwiGLU values */
@@ -486,11 +692,29 @@ __global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v)
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
 }
 
-inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles)
+inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles, int tile_m)
 {
-    int64_t m_tiles = (max_rows + BM - 1) / BM + experts;   /* each expert adds at most one partial tile */
+    int64_t m_tiles = (max_rows + tile_m - 1) / tile_m + experts;   /* each expert adds at most one partial tile */
     int64_t g = m_tiles * n_tiles;
     return (unsigned)((g + 7) / 8 * 8);
+}
+
+/* the large-tile kernel needs more dynamic LDS than the default limit: raise it once per device */
+template <int MODE, bool GMM1, int OUT_DT>
+int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
+{
+    static bool configured[64] = {};
+    const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT>);
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ZBALHIP_RT_ERROR;
+    if (!configured[dev]) {
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, D_LDS_BYTES) != hipSuccess)
+            return ZBALHIP_RT_ERROR;
+        configured[dev] = true;
+    }
+    const unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, DM);
+    grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT><<<grid, DTHREADS, D_LDS_BYTES, st>>>(p);
+    return zbalhip_check_launch();
 }
 
 } // namespace
@@ -502,7 +726,7 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
 {
     if (!a || !a_scale || !w1 || !w1scale || !row_off || !q2 || !scale2) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
-    if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || n1 <= 0 || n1 % 256 != 0)
+    if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || k > 128 * 256 || n1 <= 0 || n1 % 256 != 0)
         return ZBALHIP_INVALID;
     if (max_rows == 0) return ZBALHIP_OK;
     hipStream_t st = (hipStream_t)stream;
@@ -511,17 +735,17 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
     p.experts = (int)experts; p.max_rows = (int)max_rows; p.K = (int)k; p.N = (int)n1;
     p.out = q2; p.out_scale = scale2; p.sgl_ws = sgl_ws;
     const int n_tiles = (int)(n1 / 2 / 128);
-    const unsigned grid = grid_for(max_rows, experts, n_tiles);
-    if (mode == MODE_FP8) {
-        grouped_gemm_kernel<MODE_FP8, true, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
-        return zbalhip_check_launch();
-    }
+    if (mode == MODE_FP8) return launch_dma<MODE_FP8, true, ZDT_BF16>(p, n_tiles, st);
     if (!sgl_ws) return ZBALHIP_INVALID;
     /* the row maxima live behind the SwiGLU values in the same scratch allocation */
     p.rowmax = (uint32_t *)(sgl_ws + max_rows * (n1 / 2));
     fill_u32_kernel<<<(unsigned)((max_rows + 255) / 256), 256, 0, st>>>(p.rowmax, max_rows, 0u);
-    if (mode == MODE_W8A8) grouped_gemm_kernel<MODE_W8A8, true, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
-    else grouped_gemm_kernel<MODE_W4A8, true, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
+    if (mode == MODE_W8A8) {
+        const int32_t rc = launch_dma<MODE_W8A8, true, ZDT_BF16>(p, n_tiles, st);
+        if (rc != ZBALHIP_OK) return rc;
+    } else {
+        grouped_gemm_kernel<MODE_W4A8, true, ZDT_BF16><<<grid_for(max_rows, experts, n_tiles, BM), kThreads, 0, st>>>(p);
+    }
     int64_t rb = max_rows < 4096 ? max_rows : 4096;
     requant_rows_kernel<<<(unsigned)rb, 256, 0, st>>>(sgl_ws, p.rowmax, row_off, (int)experts, (int)(n1 / 2),
                                                     (int8_t *)q2, scale2);
@@ -536,7 +760,7 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
     if (!a || !a_scale || !w2 || !wscale || !row_off || !y) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
     if (out_dtype != ZDT_BF16 && out_dtype != ZDT_FP16) return ZBALHIP_INVALID;
-    if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || n <= 0 || n % BN != 0)
+    if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || k > 128 * 256 || n <= 0 || n % BN != 0)
         return ZBALHIP_INVALID;
     if (mode == MODE_W8A8 && wscale_dtype != ZDT_FP32 && wscale_dtype != ZDT_BF16) return ZBALHIP_INVALID;
     if (max_rows == 0) return ZBALHIP_OK;
@@ -546,16 +770,14 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
     p.experts = (int)experts; p.max_rows = (int)max_rows; p.K = (int)k; p.N = (int)n;
     p.wscale_is_bf16 = (wscale_dtype == ZDT_BF16);
     p.out = y;
-    const unsigned grid = grid_for(max_rows, experts, (int)(n / BN));
+    const int n_tiles = (int)(n / BN);
     const bool bf = out_dtype == ZDT_BF16;
-#define ZB_GO(M)                                                                            \
-    do {                                                                                    \
-        if (bf) grouped_gemm_kernel<M, false, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);      \
-        else grouped_gemm_kernel<M, false, ZDT_FP16><<<grid, kThreads, 0, st>>>(p);         \
-    } while (0)
-    if (mode == MODE_W8A8) ZB_GO(MODE_W8A8);
-    else if (mode == MODE_FP8) ZB_GO(MODE_FP8);
-    else ZB_GO(MODE_W4A8);
-#undef ZB_GO
+    if (mode == MODE_W8A8)
+        return bf ? launch_dma<MODE_W8A8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_W8A8, false, ZDT_FP16>(p, n_tiles, st);
+    if (mode == MODE_FP8)
+        return bf ? launch_dma<MODE_FP8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_FP8, false, ZDT_FP16>(p, n_tiles, st);
+    const unsigned grid = grid_for(max_rows, experts, n_tiles, BM);
+    if (bf) grouped_gemm_kernel<MODE_W4A8, false, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
+    else grouped_gemm_kernel<MODE_W4A8, false, ZDT_FP16><<<grid, kThreads, 0, st>>>(p);
     return zbalhip_check_launch();
 }
