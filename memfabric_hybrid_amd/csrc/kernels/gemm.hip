@@ -218,7 +218,13 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
                 }
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    const float left = g[i] / (1.0f + zb_expf(-g[i]));
+                    float left;
+                    if constexpr (MODE == MODE_FP8) {
+                        /* e4m3 keeps 3 mantissa bits: the hardware exp2 / reciprocal approximations (1 ulp) are ample */
+                        left = g[i] * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g[i] * -1.44269504088896341f));
+                    } else {
+                        left = g[i] / (1.0f + zb_expf(-g[i]));
+                    }
                     const float s = left * u[i];
                     sg[mt][nt][i] = s;
                     rmax[mt] = fmaxf(rmax[mt], fabsf(s));
@@ -593,12 +599,15 @@ grouped_gemm_dma_kernel(GemmParams p)
         w_sub[nt] = D_A_BYTES + r * BKB;
     }
 
+    /* a wave whose 64 rows lie past the expert's last row still moves data and meets the barriers, but skips the math */
+    const bool wave_active = row_begin + wm * 64 < row_end;
     issue(0, 0);
     for (int kb = 0; kb < KB; ++kb) {
         const int stage = kb & 1;
         __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's DMA for slab kb has landed */
         __syncthreads();                    /* ... and everybody else's; stage^1 is free again */
         if (kb + 1 < KB) issue(kb + 1, stage ^ 1);
+        if (!wave_active) continue;
         const uint8_t *sb = smem + stage * D_STAGE_BYTES;
 
         auto load_w = [&](int nt) -> i32x8 {
