@@ -32,6 +32,10 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
+# HBM bytes one GMM1 launch moves at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from two
+# `rocprofv3 --pmc` runs of this script (summary and counter calibration: profiles/moe_prefill_fp8_kernels.txt)
+GMM1_TRAFFIC_BYTES_T4096 = 3.478e9
+REDUCE_TRAFFIC_BYTES = 2.416e9  # 2.0 x 1048607 KiB + 262144 KiB (profiles/reduce_8x256MiB.txt)
 
 
 def parse():
@@ -40,7 +44,9 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--tokens", type=int, default=4096, help="development only; the reported workload is 4096")
-    ap.add_argument("--cpu-sample-tokens", type=int, default=128)
+    ap.add_argument("--cpu-sample-tokens", type=int, default=2560)
+    ap.add_argument("--workload", choices=["prefill", "reduce"], default="prefill",
+                    help="prefill = the headline MoE layer (default); reduce = the 8 x 256 MiB local reduction")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     return ap.parse_args()
 
@@ -62,6 +68,10 @@ def main():
     dev = torch.device("cuda", 0)
     buf = Buffer()
     lib = buf.lib
+    if args.workload == "reduce":
+        bench_reduce(args, torch, np, capi, buf)
+        buf.close()
+        return
 
     T, H, E, K, I = args.tokens, 7168, 32, 8, 2048
     N1 = 2 * I
@@ -162,7 +172,8 @@ def main():
     bytes_combine = rows * H * 2 + T * H * 2
     t1 = stage_ms["gmm1_swiglu_quant"] * 1e-3
     roofline = {"kernel": "grouped_gemm_kernel<fp8, gmm1>", "bound": "mfma", "achieved": flops1 / t1 / 1e12,
-                "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS, "traffic": None}
+                "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
+                "traffic": GMM1_TRAFFIC_BYTES_T4096 if T == 4096 else None}
     stages = {
         "ms": {k: round(v, 4) for k, v in stage_ms.items()},
         "gmm2_tflops": flops2 / (stage_ms["gmm2_dequant"] * 1e-3) / 1e12,
@@ -206,6 +217,61 @@ def main():
     }
     print(json.dumps(line))
     buf.close()
+
+
+def bench_reduce(args, torch, np, capi, buf):
+    """BASELINE configs[3]: one rank's reduce-scatter shard, 8 peer buffers of 256 MiB held as local HBM
+    allocations, through zbal_reduce_scatter. Algorithmic bytes = (8 + 1) x 256 MiB = 2.416 GB per launch."""
+    from memfabric_hybrid_amd.buffer import create_group, destroy_group
+    lib = buf.lib
+    R, nbytes = 8, 256 << 20
+    comm = create_group("bench_rs8", R, 0)
+    st = capi.stream_ptr()
+    results = {}
+    for name, tdt, zdt in (("bf16", torch.bfloat16, capi.DT_BF16), ("fp32", torch.float32, capi.DT_FP32)):
+        n = nbytes // torch.empty(0, dtype=tdt).element_size()
+        peers = [torch.randn(n, device="cuda", dtype=torch.float32).to(tdt) if tdt != torch.float32
+                 else torch.randn(n, device="cuda", dtype=tdt) for _ in range(R)]
+        out = torch.empty(n, device="cuda", dtype=tdt)
+        for r in range(R):
+            capi.check("window", lib.zbal_comm_register_peer_window(comm, r, peers[r].data_ptr(), nbytes))
+
+        def step():
+            capi.check("reduce_scatter", lib.zbal_reduce_scatter(peers[0].data_ptr(), out.data_ptr(), n, zdt,
+                                                                 capi.REDUCE_SUM, comm, st))
+        for _ in range(args.warmup):
+            step()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(args.steps):
+            step()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / args.steps
+        # fixed-order fp32 accumulation, one rounding: torch's sequential sum in fp32 is the same arithmetic
+        ref = peers[0].float()
+        for r in range(1, R):
+            ref = ref + peers[r].float()
+        ok = bool(torch.equal(ref.to(tdt), out))
+        results[name] = {"ms": ms, "gbs": (R + 1) * nbytes / (ms * 1e-3) / 1e9, "exact": ok}
+        # a one-input "reduction" is a plain copy of known traffic (2 x 256 MiB): the calibration point for
+        # the FETCH_SIZE / WRITE_SIZE counters
+        arr = (ctypes.c_void_p * 1)(peers[1].data_ptr())
+        capi.check("copy", lib.zbalhip_reduce(arr, 1, n, zdt, capi.REDUCE_SUM, out.data_ptr(), st))
+        torch.cuda.synchronize()
+        del peers, out, ref
+    destroy_group(comm)
+    b = results["bf16"]
+    line = {"metric": "local N-buffer reduce GB/s at 1 GPU", "value": b["gbs"], "unit": "GB/s", "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": b["ms"], "higher_is_better": True,
+            "scaling": "weak", "vs_baseline": None, "dtype": "bf16 in, fp32 accumulate, bf16 out", "data": "synthetic",
+            "config": {"workload": "local reduce-scatter shard (BASELINE configs[3])", "buffers": R,
+                       "bytes_per_buffer": nbytes},
+            "roofline": {"kernel": "reduce_kernel<bf16, sum, 8>", "bound": "hbm", "achieved": b["gbs"], "peak": PEAK_HBM_GBS,
+                         "unit": "GB/s", "frac": b["gbs"] / PEAK_HBM_GBS, "traffic": REDUCE_TRAFFIC_BYTES},
+            "cpu_baseline": None, "variants": results}
+    print(json.dumps(line))
 
 
 def plan_workspace(lib, T, H, K, E, N1, qmode):

@@ -1,0 +1,62 @@
+"""BASELINE configs[0] at seed 0 against the committed fixture (tests/golden/cfg1_seed0.json): the oracle must
+reproduce it on the CPU, and the HIP path must reproduce every bit-exact part of it on the GPU."""
+import hashlib
+import importlib.util
+import json
+import os
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+spec = importlib.util.spec_from_file_location("make_cfg1_fixture", os.path.join(HERE, "golden", "make_cfg1_fixture.py"))
+mk = importlib.util.module_from_spec(spec)
+spec.loader.exec_module(mk)
+FX = json.load(open(os.path.join(HERE, "golden", "cfg1_seed0.json")))
+
+
+def test_oracle_reproduces_fixture():
+    c = mk.cfg1_inputs()
+    for k, h in FX["inputs_sha256"].items():
+        assert mk.digest(c[k]) == h, "input generator drifted: %s" % k
+    r = mk.cfg1_oracle(c)
+    assert r["topk_idx"].tolist() == FX["topk_idx"]
+    assert r["tokens_per_expert"].tolist() == FX["tokens_per_expert"]
+    assert r["put_offset"].tolist() == FX["put_offset"]
+    for k, h in FX["sha256"].items():
+        assert mk.digest(r[k]) == h, k
+    assert sum(FX["tokens_per_expert"]) == 512 and np.allclose(np.array(FX["head"]["topk_w"]).sum(1), 1.0, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_gpu_reproduces_fixture():
+    import torch
+    from memfabric_hybrid_amd import capi
+    from memfabric_hybrid_amd.buffer import Buffer
+    from oracle import oracle as zo
+    from zbal_testlib import dev, host, max_rel_err
+    c = mk.cfg1_inputs()
+    buf = Buffer()
+    try:
+        idx, tw = buf.topk_route(dev(c["logits"]), c["K"])
+        _, _, per_expert, _, _ = buf.get_dispatch_layout(idx, c["E"])
+        q, s, recv_per_expert, h = buf.dispatch(dev(c["x"]), idx, tw, per_expert, capi.QUANT_INT8)
+        rows = c["T"] * c["K"]
+        y = torch.empty((rows, c["N"]), dtype=torch.bfloat16, device="cuda")
+        row_off = torch.cat([h["put_offset"].reshape(-1), h["total_recv"]]).contiguous()
+        assert buf.lib.zbalhip_gmm2_dequant(q.data_ptr(), s.data_ptr(), buf.prepack_weight(dev(c["w"])).data_ptr(),
+                                            dev(c["wscale"]).data_ptr(), capi.DT_FP32, row_off.data_ptr(), c["E"], rows,
+                                            c["H"], c["N"], 1, capi.DT_BF16, y.data_ptr(), capi.stream_ptr()) == 0
+        out = buf.combine(y, h, tw)
+        assert host(idx).tolist() == FX["topk_idx"]
+        assert host(per_expert).tolist() == FX["tokens_per_expert"]
+        assert host(h["put_offset"]).reshape(-1).tolist() == FX["put_offset"]
+        for name, t in (("send_token_idx", buf.send_token_idx), ("q", q), ("scale", s), ("y", y)):
+            assert mk.digest(host(t)) == FX["sha256"][name], name
+        # router weights agree to 2e-6 relative, so the combined output is compared by value
+        r = mk.cfg1_oracle(c)
+        assert np.allclose(host(tw), r["topk_w"], rtol=2e-6, atol=0)
+        assert max_rel_err(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(r["out"])) < 2e-2
+    finally:
+        torch.cuda.synchronize()
+        buf.close()
