@@ -486,9 +486,11 @@ grouped_gemm_kernel(GemmParams p)
  * K slabs go from HBM to LDS without passing through registers: every wave issues
  * global_load_lds_dwordx4, which deposits the 64 lanes' 16-byte chunks in 1 KiB of consecutive LDS
  * (lane l at +16*l). A block of 1 KiB holds 8 tile rows of 128 bytes; which global chunk a lane fetches is
- * free, so the chunk stored in slot s of row r is logical chunk s ^ ((r >> 1) & 7). With that XOR the 16
- * rows a fragment read touches (same logical chunk, 128-byte pitch) fall into 16 distinct groups of four
- * banks, which plain row-major storage would collapse onto two. Two stages of 64 KiB alternate: the slab
+ * free, so the chunk stored in slot s of row r is logical chunk s ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1).
+ * A fragment read touches 16 consecutive rows at the same logical chunk (128-byte pitch); with f every
+ * aligned run of 8 rows lands in 8 distinct 16-byte slots and the 16 rows in 16 distinct (row parity, slot)
+ * pairs, so the read is free of bank conflicts whether the LDS serves 8 or 16 lanes per pass; plain
+ * row-major storage would put all 16 rows on the same slot. Two stages of 64 KiB alternate: the slab
  * for step k+1 is in flight while step k is multiplied, with one barrier per step.
  * ------------------------------------------------------------------------------------------------------ */
 constexpr int DM = 256;
@@ -540,7 +542,7 @@ grouped_gemm_dma_kernel(GemmParams p)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const int r = 8 * (wave + 8 * i) + rr;
-            const int c = slot ^ ((r >> 1) & 7);
+            const int c = slot ^ ((r & 7) ^ ((r >> 3) & 1));
             int gr = row_begin + r;
             if (gr > p.max_rows - 1) gr = p.max_rows - 1;
             a_src[i] = p.a + (int64_t)gr * K + c * 16;
@@ -588,7 +590,7 @@ grouped_gemm_dma_kernel(GemmParams p)
 
     /* fragment reads: row lane%16 of a 16-row sub-tile, logical chunks 2*(lane/16) and 2*(lane/16)+1 */
     const int frag_row = lane & 15;
-    const int key = (lane >> 1) & 7, g2 = (lane >> 4) * 2;
+    const int key = (lane & 7) ^ ((lane >> 3) & 1), g2 = (lane >> 4) * 2;
     const int off_lo = frag_row * BKB + ((g2 ^ key) * 16), off_hi = frag_row * BKB + (((g2 + 1) ^ key) * 16);
     int w_sub[8];
 #pragma unroll
