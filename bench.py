@@ -9,7 +9,10 @@ GEMM 1 with SwiGLU + requantise, grouped GEMM 2, weighted combine), all through
 the zbal C ABI. The workload is the DeepSeek-V3-style prefill share: 4096
 tokens x hidden 7168, 32 local experts, top-8 over uniform-random logits, fp8
 e4m3 with 1x128 activation and 128x128 weight scales, intermediate 2048.
-Synthetic data, random weights.
+Synthetic data, random weights. `--workload decode` (128 tokens, W8A8, Zipf(1.2)
+expert popularity), `--workload qwen_w4a8` (16384 tokens x hidden 4096, 128
+experts, W4A8) and `--workload reduce` measure the other configurations the same
+way; the default is the headline one.
 
 Prints ONE JSON line. `value` is tokens/s of the whole step. `roofline`
 prices the dominant kernel (grouped GEMM 1) from its algorithmic FLOPs and
@@ -45,8 +48,9 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--tokens", type=int, default=4096, help="development only; the reported workload is 4096")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2560)
-    ap.add_argument("--workload", choices=["prefill", "reduce"], default="prefill",
-                    help="prefill = the headline MoE layer (default); reduce = the 8 x 256 MiB local reduction")
+    ap.add_argument("--workload", choices=["prefill", "decode", "qwen_w4a8", "reduce"], default="prefill",
+                    help="prefill = the headline fp8 MoE layer (default); decode = 128-token W8A8 layer with Zipf routing; "
+                         "qwen_w4a8 = 16384-token W4A8 layer; reduce = the 8 x 256 MiB local reduction")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     return ap.parse_args()
 
@@ -73,29 +77,65 @@ def main():
         buf.close()
         return
 
-    T, H, E, K, I = args.tokens, 7168, 32, 8, 2048
+    bench_moe(args, torch, np, capi, buf, MOE_WORKLOADS[args.workload])
+    buf.close()
+
+
+# mode: zbal_fused_deep_moe quantMode (1 = W8A8, 2 = fp8 block-scaled, 3 = W4A8)
+MOE_WORKLOADS = {
+    "prefill": dict(name="DeepSeek-V3-style prefill share (BASELINE configs[1])", T=4096, H=7168, E=32, K=8, I=2048,
+                    mode=2, zipf=None, quant="fp8 e4m3, act 1x128, weight 128x128", dtype="fp8_e4m3"),
+    "decode": dict(name="low-latency decode share (BASELINE configs[2])", T=128, H=7168, E=32, K=8, I=2048,
+                   mode=1, zipf=1.2, quant="W8A8 int8, per-token act, per-channel weight scales", dtype="int8"),
+    "qwen_w4a8": dict(name="Qwen3-MoE-style W4A8 layer (BASELINE configs[4])", T=16384, H=4096, E=128, K=8, I=1536,
+                      mode=3, zipf=None, quant="W4A8: int8 per-token act, int4 g128 weights, fp16 group scales",
+                      dtype="int8"),
+}
+
+
+def make_weights(torch, buf, dev, mode, E, k, n):
+    """Random expert weights [E, k, n] in the logical layout, their pre-packed form and scales for `mode`."""
+    if mode == 2:
+        w = torch.empty((E, k, n), device=dev, dtype=torch.float8_e4m3fn)
+        for e in range(E):
+            w[e] = (torch.randn((k, n), device=dev) * 100.0).clamp_(-448, 448).to(torch.float8_e4m3fn)
+        s = (torch.rand((E, k // 128, n // 128), device=dev) + 0.5) * (1.0 / (100.0 * k ** 0.5))
+        return w, buf.prepack_weight(w), s
+    if mode == 1:
+        w = torch.randint(-127, 128, (E, k, n), device=dev, dtype=torch.int8)
+        s = (torch.rand((E, n), device=dev) + 0.5) * (1.0 / (73.0 * k ** 0.5))
+        return w, buf.prepack_weight(w), s
+    w = torch.randint(-8, 8, (E, k, n), device=dev, dtype=torch.int8)
+    s = ((torch.rand((E, k // 128, n), device=dev) + 0.5) * (1.0 / (4.6 * k ** 0.5))).to(torch.float16)
+    return w, buf.prepack_weight(w, int4=True), s
+
+
+def bench_moe(args, torch, np, capi, buf, cfg):
+    lib = buf.lib
+    dev = torch.device("cuda", 0)
+    T = args.tokens if args.workload == "prefill" else cfg["T"]
+    H, E, K, I, mode = cfg["H"], cfg["E"], cfg["K"], cfg["I"], cfg["mode"]
     N1 = 2 * I
     rows = T * K
     torch.manual_seed(0)
     x = torch.randn((T, H), device=dev, dtype=torch.float32).to(torch.bfloat16)
-    logits = torch.rand((T, E), device=dev, dtype=torch.float32)
+    if cfg["zipf"] is None:
+        logits = torch.rand((T, E), device=dev, dtype=torch.float32)          # uniform-random logits
+    else:
+        # Zipf(s) popularity over a fixed random permutation of the experts; adding Gumbel noise to log p makes
+        # the router's top-k a draw of K distinct experts with those popularities
+        p = 1.0 / torch.arange(1, E + 1, device=dev, dtype=torch.float32) ** cfg["zipf"]
+        p = p[torch.randperm(E, device=dev)]
+        u = torch.rand((T, E), device=dev).clamp_(1e-9, 1 - 1e-9)
+        logits = (torch.log(p / p.sum())[None, :] - torch.log(-torch.log(u))).contiguous()
 
-    def fp8_weight(k, n):
-        w = torch.empty((E, k, n), device=dev, dtype=torch.float8_e4m3fn)
-        for e in range(E):
-            w[e] = (torch.randn((k, n), device=dev, dtype=torch.float32) * 100.0).clamp_(-448, 448).to(torch.float8_e4m3fn)
-        return w
-
-    w1_logical = fp8_weight(H, N1)                       # [E, K, N] as the operator API describes them
-    w2_logical = fp8_weight(I, H)
-    w1 = buf.prepack_weight(w1_logical)                  # [E, N, K] K-contiguous
-    w2 = buf.prepack_weight(w2_logical)
-    s1 = (torch.rand((E, H // 128, N1 // 128), device=dev) + 0.5) * (1.0 / (100.0 * H ** 0.5))
-    s2 = (torch.rand((E, I // 128, H // 128), device=dev) + 0.5) * (1.0 / (100.0 * I ** 0.5))
+    w1_logical, w1, s1 = make_weights(torch, buf, dev, mode, E, H, N1)       # logical = [E, K, N] of the operator API
+    w2_logical, w2, s2 = make_weights(torch, buf, dev, mode, E, I, H)
+    if mode == 1:
+        s2 = s2.to(torch.bfloat16)                                           # the reference's GMM2 scale type
     torch.cuda.synchronize()
 
-    qmode = capi.QUANT_FP8_B128
-    ws = torch.empty(buf.fused_workspace_bytes(T, H, K, E, N1, qmode), dtype=torch.uint8, device=dev)
+    ws = torch.empty(buf.fused_workspace_bytes(T, H, K, E, N1, mode), dtype=torch.uint8, device=dev)
     out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
     topk_idx = torch.empty((T, K), dtype=torch.int64, device=dev)
     topk_w = torch.empty((T, K), dtype=torch.float32, device=dev)
@@ -104,9 +144,10 @@ def main():
 
     ti = capi.tensor_info
     null = capi.TensorInfo()
+    wdt = {1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[mode]
     d = dict(x=ti(x), logits=ti(logits), idx=ti(topk_idx), w=ti(topk_w), ids=ti(ids32),
-             w1=ti(w1, dtype=capi.DT_FP8_E4M3, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s1=ti(s1),
-             w2=ti(w2, dtype=capi.DT_FP8_E4M3, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s2=ti(s2),
+             w1=ti(w1, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s1=ti(s1),
+             w2=ti(w2, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s2=ti(s2),
              out=ti(out), nums=ti(nums), ws=ti(ws))
     r = ctypes.byref
     st = capi.stream_ptr()
@@ -116,7 +157,7 @@ def main():
         ids32.copy_(topk_idx)                            # the adaptor's int64 -> int32 cast (zbal_deepep.cpp:316)
         capi.check("fused", lib.zbal_fused_deep_moe(
             r(d["x"]), r(d["ids"]), r(d["w1"]), r(d["s1"]), r(d["w2"]), r(d["s2"]), r(d["w"]), r(null), r(null), r(null),
-            r(null), r(null), r(null), r(null), r(d["out"]), r(null), r(d["nums"]), r(d["ws"]), E, qmode, 0, N1, 0, 0,
+            r(null), r(null), r(null), r(null), r(d["out"]), r(null), r(d["nums"]), r(d["ws"]), E, mode, 0, N1, 0, 0,
             buf.comm, st, 0))
 
     for _ in range(args.warmup):
@@ -132,25 +173,28 @@ def main():
     out_fused = out.clone()
 
     # ---- the same stages one by one through the inner kernel ABI, with events between them -----------------
-    off = {k: int(v) for k, v in plan_workspace(lib, T, H, K, E, N1, qmode).items()}
+    off = {k: int(v) for k, v in plan_workspace(lib, T, H, K, E, N1, mode).items()}
     base = ws.data_ptr()
     q1, xs, eidx, row_off, scratch, q2, sc2, y = (base + off[k] for k in
                                                   ("q1", "xs", "expand_idx", "row_off", "layout_scratch", "q2", "scale2", "y"))
+    sgl = base + off["sgl"] if mode != 2 else None
     names = ["route", "permute_quant", "gmm1_swiglu_quant", "gmm2_dequant", "combine"]
+    s2dt = {1: capi.DT_BF16, 2: capi.DT_FP32, 3: capi.DT_FP16}[mode]
 
     def staged(evs):
         evs[0].record()
         capi.check("route", lib.zbalhip_topk_route(logits.data_ptr(), T, E, K, topk_idx.data_ptr(), topk_w.data_ptr(), st))
         ids32.copy_(topk_idx)
         evs[1].record()
-        capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, T, H, K, E, 2,
-                                                              q1, xs, eidx, nums.data_ptr(), row_off, scratch, 50, st))
+        capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, T, H, K, E,
+                                                              2 if mode == 2 else 1, q1, xs, eidx, nums.data_ptr(), row_off,
+                                                              scratch, 50, st))
         evs[2].record()
-        capi.check("gmm1", lib.zbalhip_gmm1_swiglu_quant(q1, xs, w1.data_ptr(), s1.data_ptr(), row_off, E, rows, H, N1, 2,
-                                                         q2, sc2, None, st))
+        capi.check("gmm1", lib.zbalhip_gmm1_swiglu_quant(q1, xs, w1.data_ptr(), s1.data_ptr(), row_off, E, rows, H, N1, mode,
+                                                         q2, sc2, sgl, st))
         evs[3].record()
-        capi.check("gmm2", lib.zbalhip_gmm2_dequant(q2, sc2, w2.data_ptr(), s2.data_ptr(), capi.DT_FP32, row_off, E, rows, I,
-                                                    H, 2, capi.DT_BF16, y, st))
+        capi.check("gmm2", lib.zbalhip_gmm2_dequant(q2, sc2, w2.data_ptr(), s2.data_ptr(), s2dt, row_off, E, rows, I,
+                                                    H, mode, capi.DT_BF16, y, st))
         evs[4].record()
         capi.check("combine", lib.zbalhip_combine(y, capi.DT_BF16, row_off, 0, topk_w.data_ptr(), ids32.data_ptr(), eidx, T, H,
                                                   K, E, out.data_ptr(), st))
@@ -168,15 +212,28 @@ def main():
 
     flops1 = 2.0 * rows * H * N1
     flops2 = 2.0 * rows * I * H
-    bytes_permute = T * H * 2 + rows * (H + H // 128 * 4)
+    qbytes = rows * (H + (H // 128 * 4 if mode == 2 else 4))
+    bytes_permute = T * H * 2 + qbytes
     bytes_combine = rows * H * 2 + T * H * 2
     t1 = stage_ms["gmm1_swiglu_quant"] * 1e-3
-    roofline = {"kernel": "grouped_gemm_kernel<fp8, gmm1>", "bound": "mfma", "achieved": flops1 / t1 / 1e12,
-                "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s", "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
-                "traffic": GMM1_TRAFFIC_BYTES_T4096 if T == 4096 else None}
+    t2 = stage_ms["gmm2_dequant"] * 1e-3
+    if args.workload == "decode":
+        # a handful of rows per expert: the GEMMs stream the weights of the experts that received tokens
+        touched = int((nums > 0).sum().item())
+        wbytes1 = touched * H * N1
+        roofline = {"kernel": "grouped_gemm_dma_kernel<int8, gmm1>", "bound": "hbm", "achieved": wbytes1 / t1 / 1e9,
+                    "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": wbytes1 / t1 / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                    "experts_with_tokens": touched}
+    else:
+        kname = "grouped_gemm_dma_kernel<fp8, gmm1>" if mode == 2 else "grouped_gemm_kernel<w4a8, gmm1>"
+        roofline = {"kernel": kname, "bound": "mfma", "achieved": flops1 / t1 / 1e12,
+                    "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s" if mode == 2 else "TOP/s",
+                    "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
+                    "traffic": GMM1_TRAFFIC_BYTES_T4096 if (args.workload == "prefill" and T == 4096) else None}
     stages = {
         "ms": {k: round(v, 4) for k, v in stage_ms.items()},
-        "gmm2_tflops": flops2 / (stage_ms["gmm2_dequant"] * 1e-3) / 1e12,
+        "gmm1_tflops": flops1 / t1 / 1e12,
+        "gmm2_tflops": flops2 / t2 / 1e12,
         "permute_quant_gbs": bytes_permute / (stage_ms["permute_quant"] * 1e-3) / 1e9,
         "combine_gbs": bytes_combine / (stage_ms["combine"] * 1e-3) / 1e9,
         "permute_quant_frac_hbm": bytes_permute / (stage_ms["permute_quant"] * 1e-3) / 1e9 / PEAK_HBM_GBS,
@@ -188,20 +245,26 @@ def main():
     parity = None
     if not args.no_cpu:
         from oracle import oracle as zo
-        ts = min(args.cpu_sample_tokens, T)
-        xs_np = x[:ts].view(torch.int16).cpu().numpy().view(np.uint16)
-        ids_np = ids32[:ts].cpu().numpy()
-        w_np = topk_w[:ts].cpu().numpy()
-        w1_np = w1_logical.view(torch.uint8).cpu().numpy()
-        w2_np = w2_logical.view(torch.uint8).cpu().numpy()
-        s1_np, s2_np = s1.cpu().numpy(), s2.cpu().numpy()
+        ts = min(args.cpu_sample_tokens if args.workload == "prefill" else 128, T)
+
+        def h16(t):
+            return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+        xs_np, ids_np, w_np = h16(x[:ts]), ids32[:ts].cpu().numpy(), topk_w[:ts].cpu().numpy()
+        if mode == 2:
+            w1_np, w2_np = w1_logical.view(torch.uint8).cpu().numpy(), w2_logical.view(torch.uint8).cpu().numpy()
+            s1_np, s2_np = s1.cpu().numpy(), s2.cpu().numpy()
+        else:
+            w1_np, w2_np = w1_logical.cpu().numpy(), w2_logical.cpu().numpy()
+            s1_np = s1.cpu().numpy() if mode == 1 else h16(s1)
+            s2_np = h16(s2)
         t0 = time.perf_counter()
-        ref, _ = zo.fused_moe(xs_np, zo.DT_BF16, ids_np, w_np, w1_np, s1_np, w2_np, s2_np, E, 2)
+        ref, _ = zo.fused_moe(xs_np, zo.DT_BF16, ids_np, w_np, w1_np, s1_np, w2_np, s2_np, E, mode)
         secs = time.perf_counter() - t0
-        got = zo.bf16_to_f32(out_fused[:ts].view(torch.int16).cpu().numpy().view(np.uint16))
-        want = zo.bf16_to_f32(ref)
+        got_bits = h16(out_fused[:ts])
+        got, want = zo.bf16_to_f32(got_bits), zo.bf16_to_f32(ref)
         err = float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
-        parity = {"tokens": ts, "max_rel_err": err, "tolerance": 2e-2, "ok": bool(err < 2e-2)}
+        parity = {"tokens": ts, "max_rel_err": err, "tolerance": 2e-2, "ok": bool(err < 2e-2),
+                  "bit_exact": bool(np.array_equal(got_bits, ref))}
         cpu = {"value": ts / secs, "unit": "tokens/s", "cores": zo.num_threads(), "kind": "port",
                "sample": "first %d tokens of the same batch (%d expert rows, all %d experts' weights), %.1f s" %
                          (ts, ts * K, E, secs)}
@@ -209,14 +272,12 @@ def main():
     line = {
         "metric": "MoE layer tokens/s at 1 GPU", "value": T / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp8_e4m3", "data": "synthetic",
-        "config": {"workload": "DeepSeek-V3-style prefill share (BASELINE configs[1])", "tokens": T, "hidden": H,
-                   "experts": E, "topk": K, "intermediate": I, "quant": "fp8 e4m3, act 1x128, weight 128x128",
-                   "parallelism": "1 GPU"},
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
+        "config": {"workload": cfg["name"], "tokens": T, "hidden": H, "experts": E, "topk": K, "intermediate": I,
+                   "quant": cfg["quant"], "parallelism": "1 GPU"},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "parity": parity,
     }
     print(json.dumps(line))
-    buf.close()
 
 
 def bench_reduce(args, torch, np, capi, buf):
