@@ -506,6 +506,40 @@ __device__ __forceinline__ void dma16(const uint8_t *g, uint8_t *lds_wave_base)
                                      (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
+/*
+ * The same transfer with the address split the way the instruction wants it: a wave-uniform 64-bit base in
+ * scalar registers plus a 32-bit offset per lane, and the wave's LDS destination in M0. Spelled out because
+ * the compiler otherwise keeps a 64-bit vector address per transfer alive across the whole K loop.
+ */
+__device__ __forceinline__ void dma16_sv(const uint8_t *uniform_base, uint32_t lane_off, uint32_t lds_wave_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(lds_wave_addr), "v"(lane_off), "s"(uniform_base)
+                 : "memory", "m0");
+}
+
+__device__ __forceinline__ void dma4_sv(const float *uniform_base, uint32_t lane_off_bytes, uint32_t lds_wave_addr)
+{
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :
+                 : "s"(lds_wave_addr), "v"(lane_off_bytes), "s"(uniform_base)
+                 : "memory", "m0");
+}
+
+__device__ __forceinline__ uint32_t lds_addr(const void *p)
+{
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
+}
+
+template <typename T>
+__device__ __forceinline__ const T *uniform_ptr(const T *p)
+{
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const T *)(((uint64_t)hi << 32) | lo);
+}
+
 __device__ __forceinline__ void dma4(const float *g, float *lds_wave_base)
 {
     __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
@@ -534,29 +568,40 @@ grouped_gemm_dma_kernel(GemmParams p)
     const int KB = K / 128;
     const int I = p.N / 2;
 
-    /* DMA sources: this wave fills blocks wave + 8*i (i = 0..3) of the A tile and of the W tile */
-    const uint8_t *a_src[4];
-    const uint8_t *w_src[4];
-    {
-        const int rr = lane >> 3, slot = lane & 7;
+    /*
+     * DMA sources: this wave fills blocks wave + 8*i (i = 0..3) of the A tile and of the W tile, i.e. tile rows
+     * 64*i + r0 with r0 = 8*wave + lane/8. Addresses are a wave-uniform base (scalar registers) plus a 32-bit lane
+     * offset; the swizzled chunk c depends on r0 only, so the W offset is the same for every i and the A offsets
+     * differ only through the clamp that keeps the last tile inside the buffer.
+     */
+    const int r0 = 8 * wave + (lane >> 3);
+    const int chunk = (lane & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1));
+    const uint8_t *a_base = uniform_ptr(p.a + (int64_t)row_begin * K);
+    const int last_rel = p.max_rows - 1 - row_begin;
+    uint32_t a_off[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int r = 8 * (wave + 8 * i) + rr;
-            const int c = slot ^ ((r & 7) ^ ((r >> 3) & 1));
-            int gr = row_begin + r;
-            if (gr > p.max_rows - 1) gr = p.max_rows - 1;
-            a_src[i] = p.a + (int64_t)gr * K + c * 16;
-            int wrow;
-            if (GMM1) wrow = (r < 128) ? tc.n_tile * 128 + r : I + tc.n_tile * 128 + (r - 128);
-            else wrow = tc.n_tile * BN + r;
-            w_src[i] = p.w + ((int64_t)tc.expert * p.N + wrow) * K + c * 16;
-        }
+    for (int i = 0; i < 4; ++i) {
+        int rel = 64 * i + r0;
+        if (rel > last_rel) rel = last_rel;
+        a_off[i] = (uint32_t)rel * (uint32_t)K + chunk * 16;
     }
-    const float *sa_src = nullptr;
+    const uint32_t w_off = (uint32_t)r0 * (uint32_t)K + chunk * 16;
+    const uint8_t *w_base[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int seg;
+        if (GMM1) seg = (i < 2) ? tc.n_tile * 128 + 64 * i : I + tc.n_tile * 128 + 64 * (i - 2);
+        else seg = tc.n_tile * BN + 64 * i;
+        w_base[i] = uniform_ptr(p.w + ((int64_t)tc.expert * p.N + seg) * K);
+    }
+    const float *sa_base = uniform_ptr(p.a_scale + (int64_t)row_begin * KB);
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr(smem) + wave * 1024);          /* this wave's block 0 of stage 0 */
+    const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave & 3) * 256);
+    uint32_t sa_off = 0;
     if (MODE == MODE_FP8 && wave < 4) {
-        int gr = row_begin + wave * 64 + lane;
-        if (gr > p.max_rows - 1) gr = p.max_rows - 1;
-        sa_src = p.a_scale + (int64_t)gr * KB;
+        int rel = wave * 64 + lane;
+        if (rel > last_rel) rel = last_rel;
+        sa_off = (uint32_t)rel * (uint32_t)KB * 4u;
     }
     if (MODE == MODE_FP8) {
         /* the two weight block scales of every K slab of this tile, fetched once (visible after the first barrier) */
@@ -569,13 +614,16 @@ grouped_gemm_dma_kernel(GemmParams p)
         }
     }
 
+    /* part i of a slab's DMA: this wave's i-th block of the A tile and of the W tile (and, with part 0, the scales) */
+    auto issue_part = [&](int kb, int stage, int i) {
+        const uint32_t dst = lds0 + stage * D_STAGE_BYTES + i * 8192;
+        dma16_sv(a_base + (int64_t)kb * BKB, a_off[i], dst);
+        dma16_sv(w_base[i] + (int64_t)kb * BKB, w_off, dst + D_A_BYTES);
+        if (MODE == MODE_FP8 && i == 0 && wave < 4) dma4_sv(sa_base + kb, sa_off, lds_sa0 + stage * DM * 4);
+    };
     auto issue = [&](int kb, int stage) {
-        uint8_t *sb = smem + stage * D_STAGE_BYTES;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(a_src[i] + (int64_t)kb * BKB, sb + (wave + 8 * i) * 1024);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) dma16(w_src[i] + (int64_t)kb * BKB, sb + D_A_BYTES + (wave + 8 * i) * 1024);
-        if (MODE == MODE_FP8 && wave < 4) dma4(sa_src + kb, lds_sa + stage * DM + wave * 64);
+        for (int i = 0; i < 4; ++i) issue_part(kb, stage, i);
     };
 
     f32x4 accf[4][8];
@@ -608,8 +656,15 @@ grouped_gemm_dma_kernel(GemmParams p)
         const int stage = kb & 1;
         __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's DMA for slab kb has landed */
         __syncthreads();                    /* ... and everybody else's; stage^1 is free again */
-        if (kb + 1 < KB) issue(kb + 1, stage ^ 1);
-        if (!wave_active) continue;
+        /*
+         * The DMA of slab kb+1 is issued in four parts, spread over the first half of this step's MFMAs: a wave that
+         * pushes all of its loads at once sits in the memory pipeline's queue while the matrix unit idles.
+         */
+        const bool more = kb + 1 < KB;
+        if (!wave_active) {
+            if (more) issue(kb + 1, stage ^ 1);
+            continue;
+        }
         const uint8_t *sb = smem + stage * D_STAGE_BYTES;
 
         auto load_w = [&](int nt) -> i32x8 {
@@ -645,6 +700,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             for (int nt = 0; nt < 8; ++nt) {
                 i32x8 wf_n = wf;
                 if (nt + 1 < 8) wf_n = load_w(nt + 1);
+                if (nt < 4 && more) issue_part(kb + 1, stage ^ 1, nt);
                 const bool second = GMM1 ? (nt >= 4) : (wn == 1);
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt) {
@@ -663,6 +719,7 @@ grouped_gemm_dma_kernel(GemmParams p)
 #pragma unroll
             for (int nt = 0; nt < 8; ++nt) {
                 const i32x8 wf = load_w(nt);
+                if (nt < 4 && more) issue_part(kb + 1, stage ^ 1, nt);
                 const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt)
