@@ -146,8 +146,8 @@ def bench_moe(args, torch, np, capi, buf, cfg):
     null = capi.TensorInfo()
     wdt = {1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[mode]
     d = dict(x=ti(x), logits=ti(logits), idx=ti(topk_idx), w=ti(topk_w), ids=ti(ids32),
-             w1=ti(w1, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s1=ti(s1),
-             w2=ti(w2, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_KCONTIG), s2=ti(s2),
+             w1=ti(w1, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), s1=ti(s1),
+             w2=ti(w2, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), s2=ti(s2),
              out=ti(out), nums=ti(nums), ws=ti(ws))
     r = ctypes.byref
     st = capi.stream_ptr()

@@ -167,12 +167,16 @@ typedef struct {
  * weights in a hardware-private fractal layout made by a format-cast step
  * (test_fused_deep_moe.py:66-69); the equivalent step here is
  * zbal_moe_weight_prepack(), which turns the logical [E, K, N] row-major
- * tensor into ZBAL_WEIGHT_FORMAT_KCONTIG: [E, N, K] with K contiguous
- * (for INT4X2: [E, N, K/2] bytes; in each group of 8 consecutive k, byte b
- * holds k[b] in the low and k[b+4] in the high nibble).
+ * tensor into ZBAL_WEIGHT_FORMAT_PREPACKED, the order in which the grouped
+ * GEMM streams it (same number of bytes; K and N multiples of 128):
+ *   one byte per element: [E][N/128][K/128] blocks of 16 KiB; a block holds
+ *     128 channels x 128 K-bytes, channel r at +128*r, and within a channel
+ *     the 16-byte chunk c of its K-bytes at slot c ^ (r & 7) ^ ((r >> 3) & 1);
+ *   INT4X2: [E, N, K/2] bytes; in each group of 8 consecutive k, byte b
+ *     holds k[b] in the low and k[b+4] in the high nibble.
  */
 #define ZBAL_WEIGHT_FORMAT_ND      0 /* logical [E, K, N], N contiguous */
-#define ZBAL_WEIGHT_FORMAT_KCONTIG 1 /* [E, N, K], K contiguous         */
+#define ZBAL_WEIGHT_FORMAT_PREPACKED 1 /* made by zbal_moe_weight_prepack */
 
 /*
  * Activation quantisation modes, reference zbal_def.h:149-155 (0 and 1

@@ -105,8 +105,12 @@ ZBALHIP_API int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t 
                        void *stream);
 
 /*
- * Weight pre-pack: [E,K,N] (N contiguous) -> [E,N,K] (K contiguous);
- * to_int4 != 0 packs int8 values in [-8,7] two per byte ([E,N,K/2]).
+ * Weight pre-pack of [E,K,N] (N contiguous). One byte per element:
+ * [E][N/128][K/128] blocks of 128 channels x 128 K-bytes, channel r at +128*r
+ * with 16-byte chunk c in slot c ^ (r & 7) ^ ((r >> 3) & 1); k and n multiples
+ * of 128, pointers 16-byte aligned. to_int4 != 0 packs int8 values in [-8,7]
+ * two per byte ([E,N,K/2]). The grouped GEMMs below take `w1` / `w2` in this
+ * form.
  */
 ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int64_t k, int64_t n, int32_t to_int4, void *dst,
                                void *stream);

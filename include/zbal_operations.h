@@ -101,7 +101,7 @@ int32_t zbal_combine_low_latency(const zbal_tensor_info_t *expandX, const zbal_t
  * reference zbal_operations.h:343-354. quantMode 0 and 1 run the reference's
  * W8A8 pipeline (its kernel ignores the value); 2 = fp8 e4m3 with 1x128
  * activation scales and 128x128 weight scales; 3 = int8 activations with
- * int4 group-128 weights. Weights must be in ZBAL_WEIGHT_FORMAT_KCONTIG.
+ * int4 group-128 weights. Weights must be in ZBAL_WEIGHT_FORMAT_PREPACKED.
  * Shared-expert operands and isTensorList != 0 are rejected with -2.
  */
 int32_t zbal_fused_deep_moe(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds,
@@ -139,9 +139,10 @@ int32_t zbal_moe_topk_route(const zbal_tensor_info_t *logits, int64_t topkNum, c
 /*
  * extension: convert an expert weight tensor from ZBAL_WEIGHT_FORMAT_ND
  * ([E, K, N], N contiguous, one byte per element) to
- * ZBAL_WEIGHT_FORMAT_KCONTIG ([E, N, K]). When dst->dataType is INT4X2 the
- * source is INT8 with values in [-8, 7] and the result packs two of them per
- * byte ([E, N, K/2]; nibble order as documented for ZBAL_WEIGHT_FORMAT_KCONTIG). `dst` must not alias `src`. The
+ * ZBAL_WEIGHT_FORMAT_PREPACKED (layouts in zbal_def.h; K and N must be
+ * multiples of 128). When dst->dataType is INT4X2 the source is INT8 with
+ * values in [-8, 7] and the result packs two of them per byte. `dst` must not
+ * alias `src` and both must be 16-byte aligned. The
  * stand-in for the reference's format cast of fused-kernel weights
  * (test_fused_deep_moe.py:66-69).
  */

@@ -222,7 +222,7 @@ class Buffer:
 
     # -- fused MoE ------------------------------------------------------------------------------
     def prepack_weight(self, w, int4=False):
-        """[E,K,N] one byte per element -> the library's K-contiguous layout (the reference's format cast)."""
+        """[E,K,N] one byte per element -> the library's pre-packed layout (the reference's format cast); shape stays [E,N,K]."""
         E, K, N = w.shape
         if int4:
             dst = self._empty((E, N, K // 2), torch.uint8)
@@ -257,9 +257,9 @@ class Buffer:
         null = ctypes.byref(capi.TensorInfo())
         capi.check("zbal_fused_deep_moe", self.lib.zbal_fused_deep_moe(
             self._ti(x), self._ti(expert_ids),
-            self._ti(gmm1_permuted_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_KCONTIG),
+            self._ti(gmm1_permuted_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED),
             self._ti(gmm1_permuted_weight_scale),
-            self._ti(gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_KCONTIG), self._ti(gmm2_weight_scale),
+            self._ti(gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), self._ti(gmm2_weight_scale),
             self._ti(topk_weights), self._ti(expert_smooth_scales) if expert_smooth_scales is not None else null,
             null, null, null, null, null, null, self._ti(out), null, self._ti(token_nums), self._ti(workspace),
             num_experts, quant_mode, 0, n1, 0, 0, self.comm, capi.stream_ptr(), 0))

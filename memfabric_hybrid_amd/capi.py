@@ -24,7 +24,7 @@ REDUCE_PROD, REDUCE_SUM, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
 NO_QUANT, QUANT_INT8, QUANT_FP8_B128, QUANT_W4A8_G128 = 0, 1, 2, 3
 # zbal_backend_t
 BACKEND_GPU, BACKEND_DUMMY = 0, 1
-WEIGHT_FORMAT_ND, WEIGHT_FORMAT_KCONTIG = 0, 1
+WEIGHT_FORMAT_ND, WEIGHT_FORMAT_PREPACKED = 0, 1
 
 Z_OK, Z_ERROR, Z_INVALID_PARAM = 0, -1, -2
 Z_NOT_BOOTSTRAPPED, Z_CREATE_COMM_FAILED = -15, -16

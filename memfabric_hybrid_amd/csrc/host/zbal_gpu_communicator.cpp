@@ -390,8 +390,8 @@ public:
         ZBAL_VALIDATE_RETURN(N1 % 256 == 0 && H % 256 == 0,
                              op << " failed as gmm1HLen " << N1 << " and hidden " << H << " must be multiples of 256",
                              Z_INVALID_PARAM);
-        ZBAL_VALIDATE_RETURN(gmm1Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_KCONTIG &&
-                                 gmm2Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_KCONTIG,
+        ZBAL_VALIDATE_RETURN(gmm1Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_PREPACKED &&
+                                 gmm2Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_PREPACKED,
                              op << " failed as the weights are not pre-packed (zbal_moe_weight_prepack)", Z_INVALID_PARAM);
         const int wdt = mode == 1 ? ZBAL_DATA_TYPE_INT8 : (mode == 2 ? ZBAL_DATA_TYPE_FP8_E4M3 : ZBAL_DATA_TYPE_INT4X2);
         const int wdt_alt = mode == 2 ? ZBAL_DATA_TYPE_UINT8 : wdt;

@@ -480,8 +480,8 @@ grouped_gemm_kernel(GemmParams p)
 }
 
 /* ------------------------------------------------------------------------------------------------------
- * Large-tile kernel for the 8-bit modes (W8A8, fp8): 256 token rows x 256 channels x 128 K-bytes per
- * workgroup, eight waves in a 4 x 2 grid (same 64 x 128 wave tile as above), one workgroup per CU.
+ * Large-tile kernel for the 8-bit modes (W8A8, fp8): TM token rows x 256 channels x 128 K-bytes per
+ * workgroup, TM/64 x 2 waves (same 64 x 128 wave tile as above), one workgroup per CU.
  *
  * K slabs go from HBM to LDS without passing through registers: every wave issues
  * global_load_lds_dwordx4, which deposits the 64 lanes' 16-byte chunks in 1 KiB of consecutive LDS
@@ -490,24 +490,32 @@ grouped_gemm_kernel(GemmParams p)
  * A fragment read touches 16 consecutive rows at the same logical chunk (128-byte pitch); with f every
  * aligned run of 8 rows lands in 8 distinct 16-byte slots and the 16 rows in 16 distinct (row parity, slot)
  * pairs, so the read is free of bank conflicts whether the LDS serves 8 or 16 lanes per pass; plain
- * row-major storage would put all 16 rows on the same slot. Two stages of 64 KiB alternate: the slab
- * for step k+1 is in flight while step k is multiplied, with one barrier per step.
+ * row-major storage would put all 16 rows on the same slot.
+ *
+ * Two shapes are built. TM = 256 with two stages of 64 KiB (the slab for step k+1 is in flight while step k
+ * is multiplied) has the arithmetic intensity that many-row experts need. TM = 128 with three stages of
+ * 48 KiB is for few-row experts, where the job is to stream every weight byte once at HBM speed: it keeps
+ * two weight slabs (64 KiB) in flight per CU and skips the MFMAs of 16-row groups past the expert's end.
+ * Either way there is one barrier per step.
  * ------------------------------------------------------------------------------------------------------ */
-constexpr int DM = 256;
-constexpr int DTHREADS = 512;
-constexpr int D_A_BYTES = DM * BKB;
-constexpr int D_STAGE_BYTES = (DM + BN) * BKB;
 constexpr int D_MAX_KB = 256;                 /* K up to 32768 */
-constexpr int D_LDS_BYTES = 2 * D_STAGE_BYTES + 2 * DM * 4 + 2 * DM * 4 + 2 * D_MAX_KB * 4;
 
-__device__ __forceinline__ void dma16(const uint8_t *g, uint8_t *lds_wave_base)
-{
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                     (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
-}
+template <int TM, int NSTAGE>
+struct DmaShape {
+    static constexpr int ROW_GROUPS = TM / 64;
+    static constexpr int NW = ROW_GROUPS * 2;
+    static constexpr int THREADS = NW * 64;
+    static constexpr int A_BYTES = TM * BKB;
+    static constexpr int STAGE_BYTES = (TM + BN) * BKB;
+    static constexpr int A_PARTS = TM / 8 / NW;      /* 1 KiB blocks of the A tile per wave (4) */
+    static constexpr int W_PARTS = BN / 8 / NW;      /* 1 KiB blocks of the W tile per wave (4 or 8) */
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 2 * D_MAX_KB * 4;
+    static_assert(A_PARTS == 4 && W_PARTS % 4 == 0, "issue schedule assumes four A blocks per wave");
+    static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
+};
 
 /*
- * The same transfer with the address split the way the instruction wants it: a wave-uniform 64-bit base in
+ * One LDS-DMA transfer with the address split the way the instruction wants it: a wave-uniform 64-bit base in
  * scalar registers plus a 32-bit offset per lane, and the wave's LDS destination in M0. Spelled out because
  * the compiler otherwise keeps a 64-bit vector address per transfer alive across the whole K loop.
  */
@@ -540,39 +548,45 @@ __device__ __forceinline__ const T *uniform_ptr(const T *p)
     return (const T *)(((uint64_t)hi << 32) | lo);
 }
 
-__device__ __forceinline__ void dma4(const float *g, float *lds_wave_base)
+/* wait until at most N of this wave's vector-memory operations are outstanding (they complete in order) */
+template <int N>
+__device__ __forceinline__ void wait_vmcnt()
 {
-    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)g,
-                                     (__attribute__((address_space(3))) void *)lds_wave_base, 4, 0, 0);
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit field");
+    __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
-template <int MODE, bool GMM1, int OUT_DT>
-__global__ void __launch_bounds__(DTHREADS, 2)
+template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
+__global__ void __launch_bounds__(TM * 2, 2)      /* TM/64 x 2 waves */
 grouped_gemm_dma_kernel(GemmParams p)
 {
     static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8, "int4 weights need the register-staged kernel");
+    static_assert(NSTAGE == 2 || NSTAGE == 3, "two or three stages");
+    using S = DmaShape<TM, NSTAGE>;
+    constexpr int NW = S::NW, STAGE_BYTES = S::STAGE_BYTES, A_BYTES = S::A_BYTES, W_PARTS = S::W_PARTS;
+    constexpr bool SKIP_ROW_GROUPS = TM < 256;      /* few-row shape: leave out the MFMAs of absent 16-row groups */
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
-    float *lds_sa = reinterpret_cast<float *>(smem + 2 * D_STAGE_BYTES);   /* [2][DM] */
-    float *lds_rowmax = lds_sa + 2 * DM;                                   /* [2][DM] */
-    float *lds_sw = lds_rowmax + 2 * DM;                                   /* [2][D_MAX_KB] fp8 weight block scales */
+    float *lds_sa = reinterpret_cast<float *>(smem + NSTAGE * STAGE_BYTES);   /* [NSTAGE][TM] */
+    float *lds_rowmax = lds_sa + NSTAGE * TM;                                 /* [2][TM] */
+    float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2][D_MAX_KB] fp8 weight block scales */
 
     const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
     TileCoord tc;
-    if (!locate_tile<DM>(p.row_off, p.experts, n_tiles, tc)) return;
+    if (!locate_tile<TM>(p.row_off, p.experts, n_tiles, tc)) return;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wm = wave >> 1, wn = wave & 1;
-    const int row_begin = p.row_off[tc.expert] + tc.m_tile * DM;
+    const int row_begin = p.row_off[tc.expert] + tc.m_tile * TM;
     const int row_end = p.row_off[tc.expert + 1];
     const int K = p.K;
     const int KB = K / 128;
     const int I = p.N / 2;
 
     /*
-     * DMA sources: this wave fills blocks wave + 8*i (i = 0..3) of the A tile and of the W tile, i.e. tile rows
-     * 64*i + r0 with r0 = 8*wave + lane/8. Addresses are a wave-uniform base (scalar registers) plus a 32-bit lane
-     * offset; the swizzled chunk c depends on r0 only, so the W offset is the same for every i and the A offsets
-     * differ only through the clamp that keeps the last tile inside the buffer.
+     * DMA sources: this wave fills blocks wave + NW*j of the A tile (j < 4) and of the W tile (j < W_PARTS), i.e.
+     * tile rows 8*NW*j + r0 with r0 = 8*wave + lane/8. Addresses are a wave-uniform base (scalar registers) plus a
+     * 32-bit lane offset; the swizzled chunk depends on r0 only, so the A offsets differ only through the clamp
+     * that keeps the last tile inside the buffer.
      */
     const int r0 = 8 * wave + (lane >> 3);
     const int chunk = (lane & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1));
@@ -581,24 +595,32 @@ grouped_gemm_dma_kernel(GemmParams p)
     uint32_t a_off[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        int rel = 64 * i + r0;
+        int rel = 8 * NW * i + r0;
         if (rel > last_rel) rel = last_rel;
         a_off[i] = (uint32_t)rel * (uint32_t)K + chunk * 16;
     }
-    const uint32_t w_off = (uint32_t)r0 * (uint32_t)K + chunk * 16;
-    const uint8_t *w_base[4];
+    /*
+     * Weights come pre-packed as 16 KiB blocks of 128 channels x 128 K-bytes in LDS order ([E][N/128][K/128]):
+     * the tile's two channel halves are two such block rows, and 1 KiB block number wave + NW*j of the tile is
+     * block (wave + NW*j) % 16 of half (wave + NW*j) / 16.
+     */
+    const uint32_t w_off = lane * 16;
+    const uint8_t *w_base[W_PARTS];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int seg;
-        if (GMM1) seg = (i < 2) ? tc.n_tile * 128 + 64 * i : I + tc.n_tile * 128 + 64 * (i - 2);
-        else seg = tc.n_tile * BN + 64 * i;
-        w_base[i] = uniform_ptr(p.w + ((int64_t)tc.expert * p.N + seg) * K);
+    for (int j = 0; j < W_PARTS; ++j) {
+        const int blk = __builtin_amdgcn_readfirstlane(wave) + NW * j;
+        const int half = blk >> 4;
+        int col;                                     /* which 128-channel block row of the expert's matrix */
+        if (GMM1) col = half == 0 ? tc.n_tile : I / 128 + tc.n_tile;
+        else col = tc.n_tile * 2 + half;
+        w_base[j] = uniform_ptr(p.w + (((int64_t)tc.expert * (p.N / 128) + col) * KB) * 16384 + (blk & 15) * 1024);
     }
     const float *sa_base = uniform_ptr(p.a_scale + (int64_t)row_begin * KB);
-    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr(smem) + wave * 1024);          /* this wave's block 0 of stage 0 */
-    const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave & 3) * 256);
+    const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr(smem) + wave * 1024);     /* this wave's block 0 of stage 0 */
+    const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave % S::ROW_GROUPS) * 256);
+    const bool sa_wave = MODE == MODE_FP8 && wave < S::ROW_GROUPS;
     uint32_t sa_off = 0;
-    if (MODE == MODE_FP8 && wave < 4) {
+    if (sa_wave) {
         int rel = wave * 64 + lane;
         if (rel > last_rel) rel = last_rel;
         sa_off = (uint32_t)rel * (uint32_t)KB * 4u;
@@ -608,23 +630,25 @@ grouped_gemm_dma_kernel(GemmParams p)
         const int sw_stride = p.N / 128;
         const float *base = (const float *)p.wscale + (int64_t)tc.expert * KB * sw_stride;
         const int c0 = GMM1 ? tc.n_tile : tc.n_tile * 2, c1 = GMM1 ? I / 128 + tc.n_tile : tc.n_tile * 2 + 1;
-        for (int kb = tid; kb < KB; kb += DTHREADS) {
+        for (int kb = tid; kb < KB; kb += S::THREADS) {
             lds_sw[kb] = base[(int64_t)kb * sw_stride + c0];
             lds_sw[D_MAX_KB + kb] = base[(int64_t)kb * sw_stride + c1];
         }
     }
 
-    /* part i of a slab's DMA: this wave's i-th block of the A tile and of the W tile (and, with part 0, the scales) */
-    auto issue_part = [&](int kb, int stage, int i) {
-        const uint32_t dst = lds0 + stage * D_STAGE_BYTES + i * 8192;
-        dma16_sv(a_base + (int64_t)kb * BKB, a_off[i], dst);
-        dma16_sv(w_base[i] + (int64_t)kb * BKB, w_off, dst + D_A_BYTES);
-        if (MODE == MODE_FP8 && i == 0 && wave < 4) dma4_sv(sa_base + kb, sa_off, lds_sa0 + stage * DM * 4);
+    /* part j of a slab's DMA: this wave's j-th block of the W tile, of the A tile (j < 4) and, with part 0, the scales */
+    auto issue_part = [&](int kb, int stage, int j) {
+        const uint32_t dst = lds0 + stage * STAGE_BYTES + j * (NW * 1024);
+        dma16_sv(w_base[j] + (int64_t)kb * 16384, w_off, dst + A_BYTES);
+        if (j < 4) dma16_sv(a_base + (int64_t)kb * BKB, a_off[j], dst);
+        if (j == 0 && sa_wave) dma4_sv(sa_base + kb, sa_off, lds_sa0 + stage * TM * 4);
     };
     auto issue = [&](int kb, int stage) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) issue_part(kb, stage, i);
+        for (int j = 0; j < W_PARTS; ++j) issue_part(kb, stage, j);
     };
+    /* this wave's vector-memory operations per slab: what may stay outstanding while an older slab is awaited */
+    constexpr int OPS = W_PARTS + 4;
 
     f32x4 accf[4][8];
     i32x4 acci[4][8];
@@ -646,26 +670,45 @@ grouped_gemm_dma_kernel(GemmParams p)
         int r;
         if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
         else r = wn * 128 + nt * 16;
-        w_sub[nt] = D_A_BYTES + r * BKB;
+        w_sub[nt] = A_BYTES + r * BKB;
     }
 
     /* a wave whose 64 rows lie past the expert's last row still moves data and meets the barriers, but skips the math */
-    const bool wave_active = row_begin + wm * 64 < row_end;
-    issue(0, 0);
+    const int rows_here = row_end - (row_begin + wm * 64);
+    const bool wave_active = rows_here > 0;
+    const int mt_act = rows_here >= 64 ? 4 : (rows_here + 15) >> 4;      /* 16-row groups that hold rows */
+#pragma unroll
+    for (int s = 0; s < NSTAGE - 1; ++s)
+        if (s < KB) issue(s, s);
+    int stage = 0;
     for (int kb = 0; kb < KB; ++kb) {
-        const int stage = kb & 1;
-        __builtin_amdgcn_s_waitcnt(0x0F70); /* vmcnt(0): this wave's DMA for slab kb has landed */
-        __syncthreads();                    /* ... and everybody else's; stage^1 is free again */
+        /* this wave's DMA for slab kb has landed (later slabs may still be in flight) */
+        if (NSTAGE == 3 && kb + 1 < KB) {
+            if (sa_wave) wait_vmcnt<OPS + 1>();
+            else wait_vmcnt<OPS>();
+        } else {
+            wait_vmcnt<0>();
+        }
+        __syncthreads();                    /* ... and everybody else's; the stage read in step kb-1 is free again */
         /*
-         * The DMA of slab kb+1 is issued in four parts, spread over the first half of this step's MFMAs: a wave that
-         * pushes all of its loads at once sits in the memory pipeline's queue while the matrix unit idles.
+         * The DMA of slab kb+NSTAGE-1 goes into that stage. It is issued in parts, spread over the first half of
+         * this step's MFMAs: a wave that pushes all of its loads at once sits in the memory pipeline's queue while
+         * the matrix unit idles.
          */
-        const bool more = kb + 1 < KB;
+        const int fill_kb = kb + NSTAGE - 1;
+        const int fill_stage = stage == 0 ? NSTAGE - 1 : stage - 1;
+        const bool more = fill_kb < KB;
+        const uint8_t *sb = smem + stage * STAGE_BYTES;
+        const int cur = stage;
+        stage = stage + 1 == NSTAGE ? 0 : stage + 1;
         if (!wave_active) {
-            if (more) issue(kb + 1, stage ^ 1);
+            if (more) issue(fill_kb, fill_stage);
             continue;
         }
-        const uint8_t *sb = smem + stage * D_STAGE_BYTES;
+        auto issue_quarter = [&](int q) {
+#pragma unroll
+            for (int j = q * (W_PARTS / 4); j < (q + 1) * (W_PARTS / 4); ++j) issue_part(fill_kb, fill_stage, j);
+        };
 
         auto load_w = [&](int nt) -> i32x8 {
             const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
@@ -690,7 +733,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             float s0[4], s1[4];
 #pragma unroll
             for (int mt = 0; mt < 4; ++mt) {
-                const float sa = lds_sa[stage * DM + wm * 64 + mt * 16 + frag_row];
+                const float sa = lds_sa[cur * TM + wm * 64 + mt * 16 + frag_row];
                 s0[mt] = sa * sw0;
                 s1[mt] = sa * sw1;
             }
@@ -700,7 +743,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             for (int nt = 0; nt < 8; ++nt) {
                 i32x8 wf_n = wf;
                 if (nt + 1 < 8) wf_n = load_w(nt + 1);
-                if (nt < 4 && more) issue_part(kb + 1, stage ^ 1, nt);
+                if (nt < 4 && more) issue_quarter(nt);
                 const bool second = GMM1 ? (nt >= 4) : (wn == 1);
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt) {
@@ -719,20 +762,22 @@ grouped_gemm_dma_kernel(GemmParams p)
 #pragma unroll
             for (int nt = 0; nt < 8; ++nt) {
                 const i32x8 wf = load_w(nt);
-                if (nt < 4 && more) issue_part(kb + 1, stage ^ 1, nt);
+                if (nt < 4 && more) issue_quarter(nt);
                 const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt)
-                    acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                        wf0, i32x4{af[mt][0], af[mt][1], af[mt][2], af[mt][3]}, acci[mt][nt], 0, 0, 0);
+                    if (!SKIP_ROW_GROUPS || mt < mt_act)
+                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                            wf0, i32x4{af[mt][0], af[mt][1], af[mt][2], af[mt][3]}, acci[mt][nt], 0, 0, 0);
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt)
-                    acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                        wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
+                    if (!SKIP_ROW_GROUPS || mt < mt_act)
+                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                            wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
             }
         }
     }
-    epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, row_begin, row_end, wm, wn, lane, lds_rowmax, DM);
+    epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, row_begin, row_end, wm, wn, lane, lds_rowmax, TM);
 }
 
 /* second pass of the int8 GMM1 epilogue: whole-row requantisation from the fp32 SwiGLU values */
@@ -768,21 +813,33 @@ inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles, int til
 }
 
 /* the large-tile kernel needs more dynamic LDS than the default limit: raise it once per device */
-template <int MODE, bool GMM1, int OUT_DT>
-int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
+template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
+int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
 {
+    using S = DmaShape<TM, NSTAGE>;
     static bool configured[64] = {};
-    const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT>);
+    const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE>);
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ZBALHIP_RT_ERROR;
     if (!configured[dev]) {
-        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, D_LDS_BYTES) != hipSuccess)
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
             return ZBALHIP_RT_ERROR;
         configured[dev] = true;
     }
-    const unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, DM);
-    grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT><<<grid, DTHREADS, D_LDS_BYTES, st>>>(p);
+    const unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, TM);
+    grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE><<<grid, S::THREADS, S::LDS_BYTES, st>>>(p);
     return zbalhip_check_launch();
+}
+
+/*
+ * Shape choice from what the host knows (the row counts themselves live on the device): with at most 128 rows
+ * per expert on average the GEMM is a weight-streaming job and takes the three-stage 128-row shape.
+ */
+template <int MODE, bool GMM1, int OUT_DT>
+int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
+{
+    if ((int64_t)p.max_rows <= 128 * (int64_t)p.experts) return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
+    return launch_dma_shape<MODE, GMM1, OUT_DT, 256, 2>(p, n_tiles, st);
 }
 
 } // namespace

@@ -1,8 +1,17 @@
 /*
- * Weight pre-pack: the logical [E, K, N] byte matrix (N contiguous) becomes
- * [E, N, K] with K contiguous, the order in which the grouped GEMM streams
- * its B operand; optionally two int4 values are packed per byte. A one-time
- * step per weight tensor (64x64 tiles transposed through LDS).
+ * Weight pre-pack: the logical [E, K, N] byte matrix (N contiguous) is put
+ * into the order in which the grouped GEMM streams it. A one-time step per
+ * weight tensor.
+ *
+ * 8-bit weights: [E][N/128][K/128] blocks of 16 KiB. A block holds 128
+ * channels x 128 K-bytes exactly as the GEMM wants them in LDS: channel r of
+ * the block at +128*r, and within it the 16-byte chunk c of the K-bytes in
+ * slot c ^ f(r), f(r) = (r & 7) ^ ((r >> 3) & 1). A workgroup's weight stream
+ * is then two runs of consecutive addresses, and each LDS-DMA instruction
+ * copies 1 KiB of consecutive bytes.
+ *
+ * int4 weights: [E, N, K/2], two values per byte (64x64 tiles transposed
+ * through LDS).
  */
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
@@ -12,21 +21,27 @@ namespace {
 constexpr int kTile = 64;
 
 __global__ void __launch_bounds__(256)
-transpose_bytes_kernel(const uint8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
+tile_swizzle_bytes_kernel(const uint8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
 {
-    __shared__ uint8_t tile[kTile][kTile + 4];
+    __shared__ uint8_t tile[128][128 + 16];          /* [k][n] */
     const int64_t e = blockIdx.z;
-    const int64_t k0 = (int64_t)blockIdx.y * kTile, n0 = (int64_t)blockIdx.x * kTile;
+    const int64_t k0 = (int64_t)blockIdx.y * 128, n0 = (int64_t)blockIdx.x * 128;
     const uint8_t *s = src + e * K * N;
-    uint8_t *d = dst + e * K * N;
-    for (int i = threadIdx.x; i < kTile * kTile; i += blockDim.x) {
-        const int kk = i / kTile, nn = i % kTile;
-        if (k0 + kk < K && n0 + nn < N) tile[kk][nn] = s[(k0 + kk) * N + n0 + nn];
+    for (int i = threadIdx.x; i < 128 * 8; i += blockDim.x) {
+        const int kk = i >> 3, c = i & 7;
+        *reinterpret_cast<u32x4 *>(&tile[kk][c * 16]) = *reinterpret_cast<const u32x4 *>(s + (k0 + kk) * N + n0 + c * 16);
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < kTile * kTile; i += blockDim.x) {
-        const int nn = i / kTile, kk = i % kTile;
-        if (k0 + kk < K && n0 + nn < N) d[(n0 + nn) * K + k0 + kk] = tile[kk][nn];
+    uint8_t *d = dst + ((e * (N / 128) + blockIdx.x) * (K / 128) + blockIdx.y) * 16384;
+    for (int i = threadIdx.x; i < 1024; i += blockDim.x) {      /* one 16-byte slot per iteration */
+        const int r = i >> 3, slot = i & 7;
+        const int c = slot ^ ((r & 7) ^ ((r >> 3) & 1));
+        uint32_t w[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            w[q] = (uint32_t)tile[c * 16 + 4 * q][r] | ((uint32_t)tile[c * 16 + 4 * q + 1][r] << 8) |
+                   ((uint32_t)tile[c * 16 + 4 * q + 2][r] << 16) | ((uint32_t)tile[c * 16 + 4 * q + 3][r] << 24);
+        *reinterpret_cast<u32x4 *>(d + i * 16) = u32x4{w[0], w[1], w[2], w[3]};
     }
 }
 
@@ -64,12 +79,16 @@ extern "C" int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int6
                                           void *dst, void *stream)
 {
     if (!src || !dst || src == dst || experts <= 0 || k <= 0 || n <= 0) return ZBALHIP_INVALID;
-    if (to_int4 && (k % 8) != 0) return ZBALHIP_INVALID;
-    if (experts > 65535 || (k + kTile - 1) / kTile > 65535) return ZBALHIP_INVALID;
-    dim3 grid((unsigned)((n + kTile - 1) / kTile), (unsigned)((k + kTile - 1) / kTile), (unsigned)experts);
-    if (to_int4)
+    if (experts > 65535) return ZBALHIP_INVALID;
+    if (to_int4) {
+        if ((k % 8) != 0 || (k + kTile - 1) / kTile > 65535) return ZBALHIP_INVALID;
+        dim3 grid((unsigned)((n + kTile - 1) / kTile), (unsigned)((k + kTile - 1) / kTile), (unsigned)experts);
         transpose_pack_int4_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const int8_t *)src, k, n, (uint8_t *)dst);
-    else
-        transpose_bytes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t *)src, k, n, (uint8_t *)dst);
+    } else {
+        if ((k % 128) != 0 || (n % 128) != 0 || k / 128 > 65535) return ZBALHIP_INVALID;
+        if (((uintptr_t)src & 15) != 0 || ((uintptr_t)dst & 15) != 0) return ZBALHIP_INVALID;
+        dim3 grid((unsigned)(n / 128), (unsigned)(k / 128), (unsigned)experts);
+        tile_swizzle_bytes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t *)src, k, n, (uint8_t *)dst);
+    }
     return zbalhip_check_launch();
 }

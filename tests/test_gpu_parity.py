@@ -255,10 +255,19 @@ def test_reduce_scatter_and_all_reduce_over_peer_windows(buf):
 # ---- weight pre-pack --------------------------------------------------------------------------------------
 
 def test_weight_prepack(buf):
-    E, K, N = 3, 200, 136
+    E, K, N = 3, 256, 384
     w = rng(40).integers(-128, 128, (E, K, N)).astype(np.int8)
-    packed = buf.prepack_weight(dev(w))
-    assert np.array_equal(host(packed), np.ascontiguousarray(w.transpose(0, 2, 1)))
+    packed = host(buf.prepack_weight(dev(w))).reshape(E, N // 128, K // 128, 128, 8, 16)
+    # block [e][nb][kb] holds channel r at +128*r, 16-byte chunk c of its K-bytes in slot c ^ (r & 7) ^ ((r >> 3) & 1)
+    wt = w.transpose(0, 2, 1).reshape(E, N // 128, 128, K // 128, 8, 16).transpose(0, 1, 3, 2, 4, 5)   # [e][nb][kb][r][c][16]
+    r = np.arange(128)
+    f = (r & 7) ^ ((r >> 3) & 1)
+    want = np.empty_like(wt)
+    for slot in range(8):
+        want[:, :, :, r, slot, :] = wt[:, :, :, r, slot ^ f, :]
+    assert np.array_equal(packed, want)
+    assert buf.lib.zbalhip_weight_prepack(dev(w).data_ptr(), E, 200, 136, 0, dev(w).data_ptr() + 16, None) != 0
+    N = 136
     K = 256
     w4 = rng(41).integers(-8, 8, (E, K, N)).astype(np.int8)
     p4 = host(buf.prepack_weight(dev(w4), int4=True))
