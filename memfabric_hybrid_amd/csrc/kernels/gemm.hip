@@ -499,6 +499,7 @@ grouped_gemm_kernel(GemmParams p)
  * Either way there is one barrier per step.
  * ------------------------------------------------------------------------------------------------------ */
 constexpr int D_MAX_KB = 256;                 /* K up to 32768 */
+constexpr int D_MAX_EXPERTS = 1024;
 
 template <int TM, int NSTAGE>
 struct DmaShape {
@@ -509,7 +510,7 @@ struct DmaShape {
     static constexpr int STAGE_BYTES = (TM + BN) * BKB;
     static constexpr int A_PARTS = TM / 8 / NW;      /* 1 KiB blocks of the A tile per wave (4) */
     static constexpr int W_PARTS = BN / 8 / NW;      /* 1 KiB blocks of the W tile per wave (4 or 8) */
-    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 2 * D_MAX_KB * 4;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 4 * D_MAX_KB * 4 + 2 * (D_MAX_EXPERTS + 1) * 4;
     static_assert(A_PARTS == 4 && W_PARTS % 4 == 0, "issue schedule assumes four A blocks per wave");
     static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
 };
@@ -556,6 +557,15 @@ __device__ __forceinline__ void wait_vmcnt()
     __builtin_amdgcn_s_waitcnt(0x0F70 | (N & 15) | ((N >> 4) << 14));
 }
 
+/* what a workgroup needs to know about one tile; every member is wave-uniform and lives in scalar registers */
+struct DmaTile {
+    bool valid;
+    int expert, n_tile, row_begin, row_end, last_rel;
+    const uint8_t *a_base;            /* first K-byte of the tile's first activation row */
+    const float *sa_base;             /* its fp8 block scales */
+    const uint8_t *w_half[2];         /* K slab 0 of the tile's two 128-channel weight block rows */
+};
+
 template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
 __global__ void __launch_bounds__(TM * 2, 2)      /* TM/64 x 2 waves */
 grouped_gemm_dma_kernel(GemmParams p)
@@ -565,100 +575,155 @@ grouped_gemm_dma_kernel(GemmParams p)
     using S = DmaShape<TM, NSTAGE>;
     constexpr int NW = S::NW, STAGE_BYTES = S::STAGE_BYTES, A_BYTES = S::A_BYTES, W_PARTS = S::W_PARTS;
     constexpr bool SKIP_ROW_GROUPS = TM < 256;      /* few-row shape: leave out the MFMAs of absent 16-row groups */
+    using Tile = DmaTile;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     float *lds_sa = reinterpret_cast<float *>(smem + NSTAGE * STAGE_BYTES);   /* [NSTAGE][TM] */
     float *lds_rowmax = lds_sa + NSTAGE * TM;                                 /* [2][TM] */
-    float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2][D_MAX_KB] fp8 weight block scales */
-
-    const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
-    TileCoord tc;
-    if (!locate_tile<TM>(p.row_off, p.experts, n_tiles, tc)) return;
+    float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2 tiles][2][D_MAX_KB] fp8 weight block scales */
+    int *lds_mtp = reinterpret_cast<int *>(lds_sw + 4 * D_MAX_KB);            /* [experts + 1] tiles of TM rows before expert e */
+    int *lds_roff = lds_mtp + (D_MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wave_u = __builtin_amdgcn_readfirstlane(wave);
     const int wm = wave >> 1, wn = wave & 1;
-    const int row_begin = p.row_off[tc.expert] + tc.m_tile * TM;
-    const int row_end = p.row_off[tc.expert + 1];
+    const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
     const int K = p.K;
     const int KB = K / 128;
     const int I = p.N / 2;
+    const int E = p.experts;
 
     /*
-     * DMA sources: this wave fills blocks wave + NW*j of the A tile (j < 4) and of the W tile (j < W_PARTS), i.e.
-     * tile rows 8*NW*j + r0 with r0 = 8*wave + lane/8. Addresses are a wave-uniform base (scalar registers) plus a
-     * 32-bit lane offset; the swizzled chunk depends on r0 only, so the A offsets differ only through the clamp
-     * that keeps the last tile inside the buffer.
+     * The workgroup is persistent: it walks a fixed sequence of tiles, and the DMA runs NSTAGE-1 slabs ahead of the
+     * MFMAs across tile boundaries, so a tile's epilogue and the next tile's first loads overlap. The tile lookup
+     * tables are built once, in LDS, so that finding the next tile costs no vector-memory traffic (whose waits would
+     * also wait for the slabs in flight).
+     */
+    if (wave == 0) {
+        int run = 0;
+        for (int base = 0; base < E; base += 64) {
+            const int e = base + lane;
+            int mt = 0;
+            if (e < E) {
+                const int lo = p.row_off[e];
+                mt = (p.row_off[e + 1] - lo + TM - 1) / TM;
+                lds_roff[e] = lo;
+            }
+            int incl = mt;
+#pragma unroll
+            for (int off = 1; off < 64; off <<= 1) {
+                const int o = __shfl_up(incl, off, 64);
+                if (lane >= off) incl += o;
+            }
+            if (e < E) lds_mtp[e] = run + incl - mt;
+            run += __shfl(incl, 63, 64);
+        }
+        if (lane == 0) {
+            lds_mtp[E] = run;
+            lds_roff[E] = p.row_off[E];
+        }
+    }
+    __syncthreads();
+    /* XCD x (workgroups x, x+8, ...) owns the contiguous range [x*chunk, (x+1)*chunk) of the logical tile order */
+    const int total = __builtin_amdgcn_readfirstlane(lds_mtp[E]) * n_tiles;
+    const int chunk = (total + 7) / 8;
+    const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
+    const int lid_end = (xcd + 1) * chunk < total ? (xcd + 1) * chunk : total;
+    int lid = xcd * chunk + (blockIdx.x >> 3);
+
+    auto load_tile = [&](int id, Tile &t) {
+        t.valid = id < lid_end;
+        if (!t.valid) return;
+        const int q = id / n_tiles;                  /* index among all TM-row tiles: expert e has [mtp[e], mtp[e+1]) */
+        int expert = 0, first = 0, next = 0;
+        for (int base = 0; base < E; base += 64) {
+            const int e = base + lane;
+            int lo = 0x7fffffff, hi = 0x7fffffff;
+            if (e < E) { lo = lds_mtp[e]; hi = lds_mtp[e + 1]; }
+            const uint64_t bal = __ballot(lo <= q && q < hi);
+            if (bal) {
+                const int src = __ffsll((long long)bal) - 1;
+                expert = base + src;
+                first = __shfl(lo, src, 64);
+                next = __shfl(hi, src, 64);
+                break;
+            }
+        }
+        expert = __builtin_amdgcn_readfirstlane(expert);
+        first = __builtin_amdgcn_readfirstlane(first);
+        const int mt_e = __builtin_amdgcn_readfirstlane(next) - first;
+        /* within the expert: groups of GROUP_N channel tiles, row tiles fastest, so that concurrent tiles share slabs */
+        const int l = id - first * n_tiles;
+        const int per_group = mt_e * GROUP_N;
+        const int ng = l / per_group;
+        const int r = l - ng * per_group;
+        const int m_tile = r % mt_e;
+        t.expert = expert;
+        t.n_tile = ng * GROUP_N + r / mt_e;
+        t.row_begin = __builtin_amdgcn_readfirstlane(lds_roff[expert]) + m_tile * TM;
+        t.row_end = __builtin_amdgcn_readfirstlane(lds_roff[expert + 1]);
+        t.last_rel = t.row_end - 1 - t.row_begin;   /* rows past the expert's end re-read its last row: in bounds, and one line */
+        t.a_base = p.a + (int64_t)t.row_begin * K;
+        t.sa_base = p.a_scale + (int64_t)t.row_begin * KB;
+        /* weights come pre-packed as 16 KiB blocks of 128 channels x 128 K-bytes in LDS order ([E][N/128][K/128]) */
+        const int col0 = GMM1 ? t.n_tile : t.n_tile * 2, col1 = GMM1 ? I / 128 + t.n_tile : t.n_tile * 2 + 1;
+        t.w_half[0] = p.w + (((int64_t)expert * (p.N / 128) + col0) * KB) * 16384;
+        t.w_half[1] = p.w + (((int64_t)expert * (p.N / 128) + col1) * KB) * 16384;
+    };
+
+    /*
+     * DMA: this wave fills 1 KiB blocks wave + NW*j of the A tile (j < 4) and of the W tile (j < W_PARTS). An A block is
+     * tile rows 8*NW*j + r0 with r0 = 8*wave + lane/8, one swizzled 16-byte chunk per lane; rows past the expert's end
+     * are clamped onto its last row. 1 KiB block number b = wave + NW*j of the W tile is block b % 16 of
+     * the weight half b / 16, a straight copy. Addresses are a wave-uniform base plus a 32-bit lane offset.
      */
     const int r0 = 8 * wave + (lane >> 3);
-    const int chunk = (lane & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1));
-    const uint8_t *a_base = uniform_ptr(p.a + (int64_t)row_begin * K);
-    const int last_rel = p.max_rows - 1 - row_begin;
-    uint32_t a_off[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int rel = 8 * NW * i + r0;
-        if (rel > last_rel) rel = last_rel;
-        a_off[i] = (uint32_t)rel * (uint32_t)K + chunk * 16;
-    }
-    /*
-     * Weights come pre-packed as 16 KiB blocks of 128 channels x 128 K-bytes in LDS order ([E][N/128][K/128]):
-     * the tile's two channel halves are two such block rows, and 1 KiB block number wave + NW*j of the tile is
-     * block (wave + NW*j) % 16 of half (wave + NW*j) / 16.
-     */
-    const uint32_t w_off = lane * 16;
-    const uint8_t *w_base[W_PARTS];
-#pragma unroll
-    for (int j = 0; j < W_PARTS; ++j) {
-        const int blk = __builtin_amdgcn_readfirstlane(wave) + NW * j;
-        const int half = blk >> 4;
-        int col;                                     /* which 128-channel block row of the expert's matrix */
-        if (GMM1) col = half == 0 ? tc.n_tile : I / 128 + tc.n_tile;
-        else col = tc.n_tile * 2 + half;
-        w_base[j] = uniform_ptr(p.w + (((int64_t)tc.expert * (p.N / 128) + col) * KB) * 16384 + (blk & 15) * 1024);
-    }
-    const float *sa_base = uniform_ptr(p.a_scale + (int64_t)row_begin * KB);
+    const uint32_t a_chunk = ((lane & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1))) * 16;
+    const uint32_t w_off = wave * 1024 + lane * 16;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr(smem) + wave * 1024);     /* this wave's block 0 of stage 0 */
     const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave % S::ROW_GROUPS) * 256);
     const bool sa_wave = MODE == MODE_FP8 && wave < S::ROW_GROUPS;
-    uint32_t sa_off = 0;
-    if (sa_wave) {
-        int rel = wave * 64 + lane;
-        if (rel > last_rel) rel = last_rel;
-        sa_off = (uint32_t)rel * (uint32_t)KB * 4u;
-    }
-    if (MODE == MODE_FP8) {
-        /* the two weight block scales of every K slab of this tile, fetched once (visible after the first barrier) */
-        const int sw_stride = p.N / 128;
-        const float *base = (const float *)p.wscale + (int64_t)tc.expert * KB * sw_stride;
-        const int c0 = GMM1 ? tc.n_tile : tc.n_tile * 2, c1 = GMM1 ? I / 128 + tc.n_tile : tc.n_tile * 2 + 1;
-        for (int kb = tid; kb < KB; kb += S::THREADS) {
-            lds_sw[kb] = base[(int64_t)kb * sw_stride + c0];
-            lds_sw[D_MAX_KB + kb] = base[(int64_t)kb * sw_stride + c1];
-        }
-    }
-
-    /* part j of a slab's DMA: this wave's j-th block of the W tile, of the A tile (j < 4) and, with part 0, the scales */
-    auto issue_part = [&](int kb, int stage, int j) {
+    /* part j of a slab: the wave's j-th block of the W tile, of the A tile (j < 4) and, with part 0, the activation scales */
+    auto issue_part = [&](const Tile &t, int kb, int stage, int j) {
         const uint32_t dst = lds0 + stage * STAGE_BYTES + j * (NW * 1024);
-        dma16_sv(w_base[j] + (int64_t)kb * 16384, w_off, dst + A_BYTES);
-        if (j < 4) dma16_sv(a_base + (int64_t)kb * BKB, a_off[j], dst);
-        if (j == 0 && sa_wave) dma4_sv(sa_base + kb, sa_off, lds_sa0 + stage * TM * 4);
+        dma16_sv(t.w_half[(NW * j) >> 4] + ((int64_t)kb * 16384 + ((NW * j) & 15) * 1024), w_off, dst + A_BYTES);
+        if (j < 4) {
+            /*
+             * An 8-row block past the expert's end moves 16 bytes instead of 1 KiB (one lane): the transfer still
+             * counts as one operation of this wave, which keeps the outstanding-operation arithmetic the same for
+             * every wave and tile.
+             */
+            const bool present = 8 * NW * j + 8 * wave_u <= t.last_rel;
+            int rel = 8 * NW * j + r0;
+            if (rel > t.last_rel) rel = t.last_rel;
+            if (present || lane == 0) dma16_sv(t.a_base + (int64_t)kb * BKB, (uint32_t)rel * (uint32_t)K + a_chunk, dst);
+        }
+        if (j == 0 && sa_wave) {
+            int rel = wave * 64 + lane;
+            if (rel > t.last_rel) rel = t.last_rel;
+            dma4_sv(t.sa_base + kb, (uint32_t)rel * (uint32_t)KB * 4u, lds_sa0 + stage * TM * 4);
+        }
     };
-    auto issue = [&](int kb, int stage) {
+    auto issue = [&](const Tile &t, int kb, int stage) {
 #pragma unroll
-        for (int j = 0; j < W_PARTS; ++j) issue_part(kb, stage, j);
+        for (int j = 0; j < W_PARTS; ++j) issue_part(t, kb, stage, j);
+    };
+    /* the two weight block scales of every K slab of a tile go to LDS by DMA as well: lane = K slab */
+    auto issue_sw = [&](const Tile &t, int buf) {
+        if (MODE != MODE_FP8) return;
+        const int sw_stride = p.N / 128;
+        const float *base = (const float *)p.wscale + (int64_t)t.expert * KB * sw_stride;
+        const int c0 = GMM1 ? t.n_tile : t.n_tile * 2, c1 = GMM1 ? I / 128 + t.n_tile : t.n_tile * 2 + 1;
+        for (int b = wave_u * 64; b < KB; b += NW * 64) {
+            if (b + lane < KB) {
+                const uint32_t off = (uint32_t)(b + lane) * (uint32_t)sw_stride * 4u;
+                const uint32_t dst = lds_addr(lds_sw) + (buf * 2 * D_MAX_KB + b) * 4;
+                dma4_sv(base + c0, off, __builtin_amdgcn_readfirstlane(dst));
+                dma4_sv(base + c1, off, __builtin_amdgcn_readfirstlane(dst) + D_MAX_KB * 4);
+            }
+        }
     };
     /* this wave's vector-memory operations per slab: what may stay outstanding while an older slab is awaited */
     constexpr int OPS = W_PARTS + 4;
-
-    f32x4 accf[4][8];
-    i32x4 acci[4][8];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < 8; ++nt) {
-            accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            acci[mt][nt] = i32x4{0, 0, 0, 0};
-        }
 
     /* fragment reads: row lane%16 of a 16-row sub-tile, logical chunks 2*(lane/16) and 2*(lane/16)+1 */
     const int frag_row = lane & 15;
@@ -673,111 +738,142 @@ grouped_gemm_dma_kernel(GemmParams p)
         w_sub[nt] = A_BYTES + r * BKB;
     }
 
-    /* a wave whose 64 rows lie past the expert's last row still moves data and meets the barriers, but skips the math */
-    const int rows_here = row_end - (row_begin + wm * 64);
-    const bool wave_active = rows_here > 0;
-    const int mt_act = rows_here >= 64 ? 4 : (rows_here + 15) >> 4;      /* 16-row groups that hold rows */
+    Tile cur, nxt;
+    load_tile(lid, cur);
+    if (!cur.valid) return;
+    int sw_buf = 0;
+    issue_sw(cur, sw_buf);
 #pragma unroll
-    for (int s = 0; s < NSTAGE - 1; ++s)
-        if (s < KB) issue(s, s);
+    for (int s = 0; s < NSTAGE - 1; ++s) issue(cur, s, s);        /* the host guarantees KB >= NSTAGE - 1 */
     int stage = 0;
-    for (int kb = 0; kb < KB; ++kb) {
-        /* this wave's DMA for slab kb has landed (later slabs may still be in flight) */
-        if (NSTAGE == 3 && kb + 1 < KB) {
-            if (sa_wave) wait_vmcnt<OPS + 1>();
-            else wait_vmcnt<OPS>();
-        } else {
-            wait_vmcnt<0>();
-        }
-        __syncthreads();                    /* ... and everybody else's; the stage read in step kb-1 is free again */
-        /*
-         * The DMA of slab kb+NSTAGE-1 goes into that stage. It is issued in parts, spread over the first half of
-         * this step's MFMAs: a wave that pushes all of its loads at once sits in the memory pipeline's queue while
-         * the matrix unit idles.
-         */
-        const int fill_kb = kb + NSTAGE - 1;
-        const int fill_stage = stage == 0 ? NSTAGE - 1 : stage - 1;
-        const bool more = fill_kb < KB;
-        const uint8_t *sb = smem + stage * STAGE_BYTES;
-        const int cur = stage;
-        stage = stage + 1 == NSTAGE ? 0 : stage + 1;
-        if (!wave_active) {
-            if (more) issue(fill_kb, fill_stage);
-            continue;
-        }
-        auto issue_quarter = [&](int q) {
-#pragma unroll
-            for (int j = q * (W_PARTS / 4); j < (q + 1) * (W_PARTS / 4); ++j) issue_part(fill_kb, fill_stage, j);
-        };
+    while (true) {
+        lid += slots;
+        load_tile(lid, nxt);
+        if (nxt.valid) issue_sw(nxt, sw_buf ^ 1);   /* older than every slab issued below, so the slab waits cover it */
 
-        auto load_w = [&](int nt) -> i32x8 {
-            const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
-            const u32x4 hi = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_hi);
-            return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-        };
-        i32x8 af[4];
+        f32x4 accf[4][8];
+        i32x4 acci[4][8];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
-            const uint8_t *ab = sb + (wm * 64 + mt * 16) * BKB;
-            const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
-            const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
-            af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-        }
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int nt = 0; nt < 8; ++nt) {
+                accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+                acci[mt][nt] = i32x4{0, 0, 0, 0};
+            }
+        /* a wave whose 64 rows lie past the expert's last row still moves data and meets the barriers, but skips the math */
+        const int rows_here = cur.row_end - (cur.row_begin + wm * 64);
+        const bool wave_active = rows_here > 0;
+        const int mt_act = rows_here >= 64 ? 4 : (rows_here + 15) >> 4;      /* 16-row groups that hold rows */
+        const float *sw_cur = lds_sw + sw_buf * 2 * D_MAX_KB;
 
-        if constexpr (MODE == MODE_FP8) {
+        for (int kb = 0; kb < KB; ++kb) {
+            /* the slab after this one exists if the tile or the sequence goes on; its loads may stay in flight */
+            const bool later = kb + 1 < KB || nxt.valid;
+            if (NSTAGE == 3 && later) {
+                if (sa_wave) wait_vmcnt<OPS + 1>();
+                else wait_vmcnt<OPS>();
+            } else {
+                wait_vmcnt<0>();
+            }
+            __syncthreads();                /* slab kb has landed for everybody; the stage read in the step before is free */
             /*
-             * Software pipeline over the 32 (channel sub-tile, row sub-tile) pairs: the MFMA of pair p+1 is issued
-             * before the four scale-and-accumulate FMAs of pair p, so the vector ALU works under the matrix unit.
+             * That stage takes the slab NSTAGE-1 steps ahead, which may belong to the next tile. It is issued in parts,
+             * spread over the first half of this step's MFMAs: a wave that pushes all of its loads at once sits in the
+             * memory pipeline's queue while the matrix unit idles.
              */
-            const float sw0 = lds_sw[kb], sw1 = lds_sw[D_MAX_KB + kb];
-            float s0[4], s1[4];
+            const bool ahead_in_tile = kb + NSTAGE - 1 < KB;
+            const Tile &ft = ahead_in_tile ? cur : nxt;
+            const int fill_kb = ahead_in_tile ? kb + NSTAGE - 1 : kb + NSTAGE - 1 - KB;
+            const bool more = ahead_in_tile || nxt.valid;
+            const int fill_stage = stage == 0 ? NSTAGE - 1 : stage - 1;
+            const uint8_t *sb = smem + stage * STAGE_BYTES;
+            const int cur_stage = stage;
+            stage = stage + 1 == NSTAGE ? 0 : stage + 1;
+            if (!wave_active) {
+                if (more) issue(ft, fill_kb, fill_stage);
+                continue;
+            }
+            auto issue_quarter = [&](int q) {
+#pragma unroll
+                for (int j = q * (W_PARTS / 4); j < (q + 1) * (W_PARTS / 4); ++j) issue_part(ft, fill_kb, fill_stage, j);
+            };
+
+            auto load_w = [&](int nt) -> i32x8 {
+                const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
+                const u32x4 hi = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_hi);
+                return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+            };
+            i32x8 af[4];
 #pragma unroll
             for (int mt = 0; mt < 4; ++mt) {
-                const float sa = lds_sa[cur * TM + wm * 64 + mt * 16 + frag_row];
-                s0[mt] = sa * sw0;
-                s1[mt] = sa * sw1;
+                const uint8_t *ab = sb + (wm * 64 + mt * 16) * BKB;
+                const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
+                const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
+                af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
             }
-            i32x8 wf = load_w(0);
-            f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
-#pragma unroll
-            for (int nt = 0; nt < 8; ++nt) {
-                i32x8 wf_n = wf;
-                if (nt + 1 < 8) wf_n = load_w(nt + 1);
-                if (nt < 4 && more) issue_quarter(nt);
-                const bool second = GMM1 ? (nt >= 4) : (wn == 1);
+
+            if constexpr (MODE == MODE_FP8) {
+                /*
+                 * Software pipeline over the 32 (channel sub-tile, row sub-tile) pairs: the MFMA of pair p+1 is issued
+                 * before the four scale-and-accumulate FMAs of pair p, so the vector ALU works under the matrix unit.
+                 */
+                const float sw0 = sw_cur[kb], sw1 = sw_cur[D_MAX_KB + kb];
+                float s0[4], s1[4];
 #pragma unroll
                 for (int mt = 0; mt < 4; ++mt) {
-                    f32x4 nxt = part;
-                    if (mt < 3) nxt = mfma_fp8_16x16x128(wf, af[mt + 1]);
-                    else if (nt + 1 < 8) nxt = mfma_fp8_16x16x128(wf_n, af[0]);
-                    const float sc = second ? s1[mt] : s0[mt];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
-                    part = nxt;
+                    const float sa = lds_sa[cur_stage * TM + wm * 64 + mt * 16 + frag_row];
+                    s0[mt] = sa * sw0;
+                    s1[mt] = sa * sw1;
                 }
-                wf = wf_n;
-            }
-        } else {
-            /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
+                i32x8 wf = load_w(0);
+                f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
 #pragma unroll
-            for (int nt = 0; nt < 8; ++nt) {
-                const i32x8 wf = load_w(nt);
-                if (nt < 4 && more) issue_quarter(nt);
-                const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
+                for (int nt = 0; nt < 8; ++nt) {
+                    i32x8 wf_n = wf;
+                    if (nt + 1 < 8) wf_n = load_w(nt + 1);
+                    if (nt < 4 && more) issue_quarter(nt);
+                    const bool second = GMM1 ? (nt >= 4) : (wn == 1);
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt)
-                    if (!SKIP_ROW_GROUPS || mt < mt_act)
-                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                            wf0, i32x4{af[mt][0], af[mt][1], af[mt][2], af[mt][3]}, acci[mt][nt], 0, 0, 0);
+                    for (int mt = 0; mt < 4; ++mt) {
+                        f32x4 nxt_part = part;
+                        if (mt < 3) nxt_part = mfma_fp8_16x16x128(wf, af[mt + 1]);
+                        else if (nt + 1 < 8) nxt_part = mfma_fp8_16x16x128(wf_n, af[0]);
+                        const float sc = second ? s1[mt] : s0[mt];
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt)
-                    if (!SKIP_ROW_GROUPS || mt < mt_act)
-                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
-                            wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
+                        for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
+                        part = nxt_part;
+                    }
+                    wf = wf_n;
+                }
+            } else {
+                /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) {
+                    const i32x8 wf = load_w(nt);
+                    if (nt < 4 && more) issue_quarter(nt);
+                    const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt)
+                        if (!SKIP_ROW_GROUPS || mt < mt_act)
+                            acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                                wf0, i32x4{af[mt][0], af[mt][1], af[mt][2], af[mt][3]}, acci[mt][nt], 0, 0, 0);
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt)
+                        if (!SKIP_ROW_GROUPS || mt < mt_act)
+                            acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
+                                wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
+                }
             }
         }
+        TileCoord tc;
+        tc.expert = cur.expert;
+        tc.m_tile = 0;
+        tc.n_tile = cur.n_tile;
+        epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane, lds_rowmax, TM);
+        if (!nxt.valid) break;
+        cur = nxt;
+        sw_buf ^= 1;
     }
-    epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, row_begin, row_end, wm, wn, lane, lds_rowmax, TM);
 }
 
 /* second pass of the int8 GMM1 epilogue: whole-row requantisation from the fp32 SwiGLU values */
@@ -812,33 +908,42 @@ inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles, int til
     return (unsigned)((g + 7) / 8 * 8);
 }
 
-/* the large-tile kernel needs more dynamic LDS than the default limit: raise it once per device */
+/*
+ * The large-tile kernel needs more dynamic LDS than the default limit (raised once per device) and is launched
+ * with one persistent workgroup per CU, or fewer when there are not that many tiles.
+ */
 template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
 int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
 {
     using S = DmaShape<TM, NSTAGE>;
-    static bool configured[64] = {};
+    static int cus[64] = {};
     const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE>);
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ZBALHIP_RT_ERROR;
-    if (!configured[dev]) {
+    if (cus[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return ZBALHIP_RT_ERROR;
         if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
             return ZBALHIP_RT_ERROR;
-        configured[dev] = true;
+        cus[dev] = n;
     }
-    const unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, TM);
+    unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, TM);
+    const unsigned resident = (unsigned)(cus[dev] + 7) / 8 * 8;
+    if (grid > resident) grid = resident;
     grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE><<<grid, S::THREADS, S::LDS_BYTES, st>>>(p);
     return zbalhip_check_launch();
 }
 
 /*
  * Shape choice from what the host knows (the row counts themselves live on the device): with at most 128 rows
- * per expert on average the GEMM is a weight-streaming job and takes the three-stage 128-row shape.
+ * per expert on average the GEMM is a weight-streaming job and takes the three-stage 128-row shape, which needs
+ * two K slabs to fill its pipeline.
  */
 template <int MODE, bool GMM1, int OUT_DT>
 int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
 {
-    if ((int64_t)p.max_rows <= 128 * (int64_t)p.experts) return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
+    if ((int64_t)p.max_rows <= 128 * (int64_t)p.experts && p.K >= 256)
+        return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
     return launch_dma_shape<MODE, GMM1, OUT_DT, 256, 2>(p, n_tiles, st);
 }
 
