@@ -12,13 +12,9 @@
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
 
-int32_t zbalhip_layout_internal(const void *idx, int32_t idx_is_i64, int64_t tokens, int64_t experts, int64_t topk,
-                                int32_t ranks, int32_t *tokens_per_rank, int32_t *send_token_idx, int32_t *scratch,
-                                int max_blocks, int *nblk_out, hipStream_t st);
-int32_t zbalhip_scan_internal(const int32_t *hist, int nblk, int64_t experts, int64_t topk, int32_t token_nums_type,
-                              int32_t *counts_i32, int32_t *excl_i32, int32_t *incl_i32, int32_t *row_off,
-                              int64_t *counts_i64, int64_t *nums_typed, int32_t *total, int32_t *balance,
-                              hipStream_t st);
+int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
+                                      int32_t token_nums_type, int32_t *send_token_idx, int32_t *incl_i32,
+                                      int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed, hipStream_t st);
 
 namespace {
 
@@ -303,12 +299,8 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
         scratch_blocks < 1)
         return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
-    int nblk = 0;
-    int32_t rc = zbalhip_layout_internal(expert_ids, 0, tokens, experts, topk, 1, nullptr, expand_idx, scratch,
-                                         scratch_blocks, &nblk, st);
-    if (rc != ZBALHIP_OK) return rc;
-    rc = zbalhip_scan_internal(scratch, nblk, experts, topk, token_nums_type, nullptr, nullptr, ep_recv_counts, nullptr,
-                               nullptr, expert_token_nums, nullptr, nullptr, st);
+    const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, token_nums_type, expand_idx,
+                                                     ep_recv_counts, nullptr, nullptr, expert_token_nums, st);
     if (rc != ZBALHIP_OK) return rc;
     const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_NOEPS : QM_FP8);
     return zbalhip_permute_internal(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk,
@@ -326,12 +318,8 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
         return ZBALHIP_INVALID;
     if (mode == 2 && smooth) return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
-    int nblk = 0;
-    int32_t rc = zbalhip_layout_internal(expert_ids, 0, tokens, experts, topk, 1, nullptr, expand_idx, scratch,
-                                         scratch_blocks, &nblk, st);
-    if (rc != ZBALHIP_OK) return rc;
-    rc = zbalhip_scan_internal(scratch, nblk, experts, topk, 1, nullptr, nullptr, nullptr, row_off, counts, nullptr,
-                               nullptr, nullptr, st);
+    const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, 1, expand_idx, nullptr, row_off,
+                                                     counts, nullptr, st);
     if (rc != ZBALHIP_OK) return rc;
     return zbalhip_permute_internal(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk,
                                     experts, mode == 2 ? QM_FP8 : QM_INT8_NOEPS, q1, xs, st);

@@ -17,6 +17,7 @@
 
 #define ZB_MAX_EXPERTS 1024
 #define ZB_LAYOUT_THREADS 256
+#define ZB_FUSED_THREADS 1024
 
 namespace {
 
@@ -61,6 +62,47 @@ layout_hist_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
     for (int e = threadIdx.x; e < experts; e += blockDim.x) scratch[(int64_t)blockIdx.x * experts + e] = hist[e];
 }
 
+/*
+ * Stable ranks of the picks [p0, p1) of one block: `run[e]` holds the number of earlier picks of expert e on entry
+ * and the number up to p1 on return. Picks are taken 64 per wave at a time; lanes holding the same expert find
+ * each other by intersecting one ballot per index bit, and the waves of the block commit in wave order.
+ */
+template <typename IdxT>
+__device__ __forceinline__ void rank_picks(const IdxT *__restrict__ idx, int64_t p0, int64_t p1, int experts, int nbits,
+                                           int32_t *run, int32_t *__restrict__ send_token_idx)
+{
+    const int np = (int)(p1 - p0);
+    const int threads = blockDim.x;
+    const int iters = (np + threads - 1) / threads;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+
+    for (int it = 0; it < iters; ++it) {
+        const int64_t i = p0 + (int64_t)it * threads + threadIdx.x;
+        int64_t e64 = (i < p1) ? (int64_t)idx[i] : -1;
+        const bool valid = (e64 >= 0 && e64 < experts);
+        const int e = valid ? (int)e64 : 0;
+        uint64_t peers = __ballot(valid);
+        for (int bit = 0; bit < nbits; ++bit) {
+            const bool one = (e >> bit) & 1;
+            const uint64_t bal = __ballot(valid && one);
+            peers &= one ? bal : ~bal;
+        }
+        const int before = __popcll(peers & lt_mask);
+        const int group = __popcll(peers);
+        const bool last = valid && ((peers >> lane) >> 1) == 0; /* highest lane of its group */
+        for (int w = 0; w < (threads >> 6); ++w) {
+            if (wave == w && valid) {
+                const int32_t basev = run[e];
+                send_token_idx[i] = basev + before;
+                if (last) run[e] = basev + group;
+            }
+            __syncthreads();
+        }
+        if (!valid && i < p1) send_token_idx[i] = -1;
+    }
+}
+
 template <typename IdxT>
 __global__ void __launch_bounds__(ZB_LAYOUT_THREADS)
 layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int experts, int ranks, int tpb, int nbits,
@@ -81,36 +123,7 @@ layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
     const int tok0 = b * tpb;
     int tok1 = tok0 + tpb;
     if (tok1 > tokens) tok1 = tokens;
-    const int64_t p0 = (int64_t)tok0 * topk, p1 = (int64_t)tok1 * topk;
-    const int np = (int)(p1 - p0);
-    const int iters = (np + ZB_LAYOUT_THREADS - 1) / ZB_LAYOUT_THREADS;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-
-    for (int it = 0; it < iters; ++it) {
-        const int64_t i = p0 + (int64_t)it * ZB_LAYOUT_THREADS + threadIdx.x;
-        int64_t e64 = (i < p1) ? (int64_t)idx[i] : -1;
-        const bool valid = (e64 >= 0 && e64 < experts);
-        const int e = valid ? (int)e64 : 0;
-        uint64_t peers = __ballot(valid);
-        for (int bit = 0; bit < nbits; ++bit) {
-            const bool one = (e >> bit) & 1;
-            const uint64_t bal = __ballot(valid && one);
-            peers &= one ? bal : ~bal;
-        }
-        const int before = __popcll(peers & lt_mask);
-        const int group = __popcll(peers);
-        const bool last = valid && ((peers >> lane) >> 1) == 0; /* highest lane of its group */
-        for (int w = 0; w < ZB_LAYOUT_THREADS / 64; ++w) {
-            if (wave == w && valid) {
-                const int32_t basev = run[e];
-                send_token_idx[i] = basev + before;
-                if (last) run[e] = basev + group;
-            }
-            __syncthreads();
-        }
-        if (!valid && i < p1) send_token_idx[i] = -1;
-    }
+    rank_picks(idx, (int64_t)tok0 * topk, (int64_t)tok1 * topk, experts, nbits, run, send_token_idx);
 
     /* tokens per rank: one count per (token, rank) no matter how many of the token's picks land there */
     if (tokens_per_rank) {
@@ -131,6 +144,77 @@ layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
         __syncthreads();
         for (int r = threadIdx.x; r < ranks; r += blockDim.x)
             if (rcnt[r]) atomicAdd(&tokens_per_rank[r], rcnt[r]);
+    }
+}
+
+/*
+ * The whole layout in one launch, for the callers that need ranks and offsets but no per-rank counts: every
+ * block first counts the picks that precede its own range (the index array is a few hundred KiB and sits in L2,
+ * so reading it again per block is cheaper than a launch), ranks its own picks, and the last block, whose running
+ * counts are then the totals, scans them into the offsets. Every output pointer except send_token_idx may be null.
+ */
+template <typename IdxT>
+__global__ void __launch_bounds__(ZB_FUSED_THREADS)
+layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int experts, int tpb, int nbits,
+                    int token_nums_type, int32_t *__restrict__ send_token_idx, int32_t *__restrict__ incl_i32,
+                    int32_t *__restrict__ row_off /* [E+1] */, int64_t *__restrict__ counts_i64,
+                    int64_t *__restrict__ nums_typed)
+{
+    __shared__ int32_t run[ZB_MAX_EXPERTS];
+    __shared__ int32_t wsum[ZB_FUSED_THREADS / 64];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) run[e] = 0;
+    __syncthreads();
+    const int tok0 = blockIdx.x * tpb;
+    int tok1 = tok0 + tpb;
+    if (tok1 > tokens) tok1 = tokens;
+    const int64_t p0 = (int64_t)tok0 * topk, p1 = (int64_t)tok1 * topk;
+    constexpr int PER = 16 / (int)sizeof(IdxT);      /* indices per 16-byte load */
+    const int64_t nvec = ((uintptr_t)idx & 15) == 0 ? p0 / PER : 0;
+    for (int64_t v = threadIdx.x; v < nvec; v += blockDim.x) {
+        const u32x4 raw = *reinterpret_cast<const u32x4 *>(idx + v * PER);
+#pragma unroll
+        for (int j = 0; j < PER; ++j) {
+            int64_t e;
+            if (sizeof(IdxT) == 4) e = (int32_t)raw[j];
+            else e = (int64_t)(((uint64_t)raw[2 * j + 1] << 32) | raw[2 * j]);
+            if (e >= 0 && e < experts) atomicAdd(&run[(int)e], 1);
+        }
+    }
+    for (int64_t i = nvec * PER + threadIdx.x; i < p0; i += blockDim.x) {
+        const int64_t e = (int64_t)idx[i];
+        if (e >= 0 && e < experts) atomicAdd(&run[(int)e], 1);
+    }
+    __syncthreads();
+    rank_picks(idx, p0, p1, experts, nbits, run, send_token_idx);
+    if (blockIdx.x != gridDim.x - 1) return;
+
+    /* rank_picks ends on a barrier: run[] now holds the totals */
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    int32_t carry = 0;
+    for (int base = 0; base < experts; base += ZB_FUSED_THREADS) {
+        const int e = base + threadIdx.x;
+        const int32_t c = e < experts ? run[e] : 0;
+        int32_t s = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int32_t o = __shfl_up(s, off, 64);
+            if (lane >= off) s += o;
+        }
+        if (lane == 63) wsum[wave] = s;
+        __syncthreads();
+        int32_t add = carry;
+        for (int w = 0; w < wave; ++w) add += wsum[w];
+        s += add;
+        int32_t chunk_total = 0;
+        for (int w = 0; w < ZB_FUSED_THREADS / 64; ++w) chunk_total += wsum[w];
+        carry += chunk_total;
+        __syncthreads();
+        if (e < experts) {
+            if (incl_i32) incl_i32[e] = s;
+            if (row_off) { row_off[e] = s - c; if (e == experts - 1) row_off[experts] = s; }
+            if (counts_i64) counts_i64[e] = c;
+            if (nums_typed) nums_typed[e] = token_nums_type == 0 ? (int64_t)s : (int64_t)c;
+        }
     }
 }
 
@@ -276,6 +360,19 @@ int32_t zbalhip_layout_internal(const void *idx, int32_t idx_is_i64, int64_t tok
             send_token_idx, tokens_per_rank);
     }
     *nblk_out = p.nblk;
+    return zbalhip_check_launch();
+}
+
+/* ranks + offsets in one launch (no per-rank counts, no scratch) */
+int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
+                                      int32_t token_nums_type, int32_t *send_token_idx, int32_t *incl_i32,
+                                      int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed, hipStream_t st)
+{
+    const LayoutPlan p = plan_layout(tokens, topk, 64);
+    layout_fused_kernel<int32_t><<<p.nblk, ZB_FUSED_THREADS, 0, st>>>(idx, (int)tokens, (int)topk, (int)experts,
+                                                                    p.tokens_per_block, ceil_log2(experts), token_nums_type,
+                                                                    send_token_idx, incl_i32, row_off, counts_i64,
+                                                                    nums_typed);
     return zbalhip_check_launch();
 }
 
