@@ -84,8 +84,9 @@ ZBALHIP_API int32_t zbalhip_combine(const void *y, int32_t dtype, const int32_t 
  * quantising permute in one call. quant_mode 1 uses s = 127/amax (an
  * all-zero row gives q = 0, scale = 0). ep_recv_counts [E] = inclusive
  * running sum; expert_token_nums [E] i64 = counts (type 1) or the running
- * sum (type 0). scratch holds scratch_blocks * experts i32 (scratch_blocks
- * >= 1 bounds the number of workgroups of the layout pass).
+ * sum (type 0). scratch (scratch_blocks * experts i32, scratch_blocks >= 1)
+ * mirrors the reference's putOffset operand; the layout is computed in one
+ * launch that does not touch it.
  */
 ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, const int32_t *expert_ids, int64_t tokens,
                                      int64_t hidden, int64_t topk, int64_t experts, int32_t quant_mode,
@@ -121,7 +122,8 @@ ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int
  * 952-995, 1859-2058). mode 1: int8, s = 127/amax, optional smooth [E,H]
  * fp32 multiplied in first; mode 2: e4m3 1x128. Outputs q1 [rows,H], xs
  * ([rows] or [rows,H/128]), expand_idx [T,K], counts [E] i64 and the
- * exclusive row offsets row_off [E+1] i32. scratch / scratch_blocks as above.
+ * exclusive row offsets row_off [E+1] i32. scratch / scratch_blocks as above
+ * (not touched).
  */
 ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids, const float *smooth,
                                     int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int32_t mode,
