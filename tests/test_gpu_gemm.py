@@ -275,6 +275,87 @@ def test_fused_moe_fp8(buf, T, H, K, E, I):
     assert calc_diff(f, r) < 1e-4
 
 
+def test_prefill_share_full_size_sampled_tokens(buf):
+    """The fp8 prefill share at its real size (4096 tokens x 7168, 32 experts, top-8, intermediate 2048). A token's
+    output depends on its own row only (per-token quantisation, row-wise GEMMs, per-token combine), so the oracle is run
+    on tokens sampled across the whole batch, with the same routing, and compared with the rows of the full launch."""
+    T, H, K, E, I = 4096, 7168, 8, 32, 2048
+    g = torch.Generator(device="cuda").manual_seed(11)
+    x = torch.randn((T, H), device="cuda", generator=g).to(torch.bfloat16)
+    logits = torch.rand((T, E), device="cuda", generator=g)
+    ids, es = buf.topk_route(logits, K)
+
+    def weights(k, n):
+        w = torch.empty((E, k, n), device="cuda", dtype=torch.float8_e4m3fn)
+        for e in range(E):
+            w[e] = (torch.randn((k, n), device="cuda", generator=g) * 100.0).clamp_(-448, 448).to(torch.float8_e4m3fn)
+        sc = (torch.rand((E, k // 128, n // 128), device="cuda", generator=g) + 0.5) / (100.0 * k ** 0.5)
+        return w, sc
+    w1, s1 = weights(H, 2 * I)
+    w2, s2 = weights(I, H)
+    out, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1), s1, buf.prepack_weight(w2), s2, es, E, quant_mode=2)
+    torch.cuda.synchronize()
+    ids_h = host(ids)
+    assert np.array_equal(host(nums), np.bincount(ids_h.ravel(), minlength=E))
+    pick = np.sort(rng(12).choice(T, size=96, replace=False))
+    ref, _ = zo.fused_moe(host(x.view(torch.int16)).view(np.uint16)[pick], zo.DT_BF16, ids_h[pick], host(es)[pick],
+                          host(w1.view(torch.uint8)), host(s1), host(w2.view(torch.uint8)), host(s2), E, 2)
+    got = zo.bf16_to_f32(host(out.view(torch.int16)).view(np.uint16)[pick])
+    assert max_rel_err(got, zo.bf16_to_f32(ref)) < 2e-2
+
+
+def _int_weights(g, mode, E, k, n):
+    """Random expert weights on the GPU in the logical [E, k, n] layout, and scales, for an int mode."""
+    if mode == 3:
+        w = torch.randint(-8, 8, (E, k, n), device="cuda", dtype=torch.int8, generator=g)
+        sc = ((torch.rand((E, k // 128, n), device="cuda", generator=g) + 0.5) / (4.6 * k ** 0.5)).to(torch.float16)
+    else:
+        w = torch.randint(-127, 128, (E, k, n), device="cuda", dtype=torch.int8, generator=g)
+        sc = (torch.rand((E, n), device="cuda", generator=g) + 0.5) / (73.0 * k ** 0.5)
+    return w, sc
+
+
+def _bits16(t):
+    return host(t.contiguous().view(torch.int16)).view(np.uint16)
+
+
+def test_decode_share_full_size_bit_exact(buf):
+    """The W8A8 decode share at its real size (128 tokens x 7168, 32 experts, top-8 under Zipf(1.2) popularity,
+    intermediate 2048): every token against the oracle, bit for bit. Most experts receive a handful of rows."""
+    T, H, K, E, I = 128, 7168, 8, 32, 2048
+    g = torch.Generator(device="cuda").manual_seed(21)
+    x = torch.randn((T, H), device="cuda", generator=g).to(torch.bfloat16)
+    ids = dev(distinct_topk(T, E, K, 22, zipf=1.2))
+    es = torch.rand((T, K), device="cuda", generator=g) + 0.1
+    es = es / es.sum(dim=1, keepdim=True)
+    w1, s1 = _int_weights(g, 1, E, H, 2 * I)
+    w2, s2 = _int_weights(g, 1, E, I, H)
+    s2 = s2.to(torch.bfloat16)
+    out, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1), s1, buf.prepack_weight(w2), s2, es, E, quant_mode=1)
+    ref, counts = zo.fused_moe(_bits16(x), zo.DT_BF16, host(ids), host(es), host(w1), host(s1), host(w2), _bits16(s2), E, 1)
+    assert np.array_equal(host(nums), counts)
+    assert np.array_equal(_bits16(out), ref)
+
+
+def test_w4a8_layer_full_size_sampled_tokens_bit_exact(buf):
+    """The W4A8 layer at its real size (16384 tokens x 4096, 128 experts, top-8, intermediate 1536): the oracle is run on
+    tokens sampled across the batch (a token's output depends on its own row only) and must match bit for bit."""
+    T, H, K, E, I = 16384, 4096, 8, 128, 1536
+    g = torch.Generator(device="cuda").manual_seed(31)
+    x = torch.randn((T, H), device="cuda", generator=g).to(torch.bfloat16)
+    ids, es = buf.topk_route(torch.rand((T, E), device="cuda", generator=g), K)
+    w1, s1 = _int_weights(g, 3, E, H, 2 * I)
+    w2, s2 = _int_weights(g, 3, E, I, H)
+    out, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1, int4=True), s1, buf.prepack_weight(w2, int4=True), s2, es, E,
+                                   quant_mode=3)
+    ids_h = host(ids)
+    assert np.array_equal(host(nums), np.bincount(ids_h.ravel(), minlength=E))
+    pick = np.sort(rng(32).choice(T, size=64, replace=False))
+    ref, _ = zo.fused_moe(_bits16(x)[pick], zo.DT_BF16, ids_h[pick], host(es)[pick], host(w1), _bits16(s1), host(w2), _bits16(s2),
+                          E, 3)
+    assert np.array_equal(_bits16(out)[pick], ref)
+
+
 def test_fused_moe_empty_experts_and_invalid_ids(buf):
     T, H, K, E, I = 16, 256, 2, 32, 128                  # 32 picks over 32 experts: most experts are empty
     x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, 0, 90, zipf=1.2)

@@ -214,6 +214,31 @@ def test_reduce_kernel_all_types(buf, dt, op):
         assert np.array_equal(host(out), ref), (N, n)
 
 
+def test_reduce_full_size_sampled_windows(buf):
+    """8 buffers of 256 MiB in separate allocations, bf16 and fp32 sums: the output is checked on windows sampled at the
+    ends and across the range (the reduction is element-wise, so a window needs only the same window of every input)."""
+    lib = buf.lib
+    N, nbytes = 8, 256 << 20
+    g = torch.Generator(device="cuda").manual_seed(5)
+    for dt, tdt in ((capi.DT_BF16, torch.bfloat16), (capi.DT_FP32, torch.float32)):
+        n = nbytes // (2 if dt == capi.DT_BF16 else 4)
+        ins = [torch.randn(n, device="cuda", generator=g).to(tdt) for _ in range(N)]
+        out = torch.empty_like(ins[0])
+        arr = (ctypes.c_void_p * N)(*[t.data_ptr() for t in ins])
+        assert lib.zbalhip_reduce(arr, N, n, dt, capi.REDUCE_SUM, out.data_ptr(), capi.stream_ptr()) == 0
+        torch.cuda.synchronize()
+        w = 1 << 16
+        for start in [0, n - w] + [int(v) for v in rng(6).integers(0, n - w, 6)]:
+            if dt == capi.DT_BF16:
+                parts = [host(t[start:start + w].view(torch.int16)).view(np.uint16) for t in ins]
+                got = host(out[start:start + w].view(torch.int16)).view(np.uint16)
+            else:
+                parts = [host(t[start:start + w]) for t in ins]
+                got = host(out[start:start + w])
+            assert np.array_equal(got, zo.reduce(parts, dt, capi.REDUCE_SUM)), (dt, start)
+        del ins, out
+
+
 def test_reduce_scatter_and_all_reduce_over_peer_windows(buf):
     """cfg4 shape in miniature: 8 'ranks' as local windows, this rank reduces its slice of every peer's buffer."""
     from memfabric_hybrid_amd.buffer import create_group, destroy_group
