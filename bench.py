@@ -360,7 +360,7 @@ def plan_workspace(lib, T, H, K, E, N1, qmode):
     if not fp8:
         take("sgl", rows * (I + 1) * 4)
     take("y", rows * H * 2)
-    assert cur == lib.zbal_fused_deep_moe_workspace_size(T, H, K, E, N1, qmode), "workspace plan out of sync"
+    assert cur == lib.zbal_fused_deep_moe_workspace_size(T, H, K, E, N1, 0, qmode), "workspace plan out of sync"
     return off
 
 

@@ -105,6 +105,9 @@ ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype,
 ZBALHIP_API int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t count, int32_t dtype, int32_t op, void *out,
                        void *stream);
 
+/* p[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node) */
+ZBALHIP_API int32_t zbalhip_fill_i32(int32_t *p, int64_t n, int32_t value, void *stream);
+
 /*
  * Weight pre-pack of [E,K,N] (N contiguous). One byte per element:
  * [E][N/128][K/128] blocks of 128 channels x 128 K-bytes, channel r at +128*r

@@ -102,7 +102,13 @@ int32_t zbal_combine_low_latency(const zbal_tensor_info_t *expandX, const zbal_t
  * W8A8 pipeline (its kernel ignores the value); 2 = fp8 e4m3 with 1x128
  * activation scales and 128x128 weight scales; 3 = int8 activations with
  * int4 group-128 weights. Weights must be in ZBAL_WEIGHT_FORMAT_PREPACKED.
- * Shared-expert operands and isTensorList != 0 are rejected with -2.
+ * The shared expert (EXEC_FLAG_SHARED_EXPERT in the reference kernel,
+ * zbal_kernel_fused_deep_moe.h:470-472) is one more expert applied to every
+ * token: shareGmm1Weight [H, shareGmm1HLen] and shareGmm2Weight
+ * [shareGmm1HLen/2, H] pre-packed like the others, scales shaped as one
+ * expert's, optional shareSmoothScales [H]; its result goes to shareOutput
+ * [tokens, H] and is not added to output. Pass all of them or none.
+ * xActiveMask and isTensorList != 0 are rejected with -2.
  */
 int32_t zbal_fused_deep_moe(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds,
                             const zbal_tensor_info_t *gmm1Weight, const zbal_tensor_info_t *gmm1Scale,
@@ -121,10 +127,11 @@ int32_t zbal_fused_deep_moe(const zbal_tensor_info_t *x, const zbal_tensor_info_
  * extension: bytes of workspace zbal_fused_deep_moe needs for a batch of
  * `tokens` rows. Takes the place of the size computation the reference keeps
  * in its adaptor and host launcher (zbal_deepep.cpp:42-84,
- * zbal_kernel_fused_deep_moe_host.cpp:59-132). Returns 0 on invalid input.
+ * zbal_kernel_fused_deep_moe_host.cpp:59-132). shareGmm1HLen is 0 without a
+ * shared expert. Returns 0 on invalid input.
  */
 uint64_t zbal_fused_deep_moe_workspace_size(int64_t tokens, int64_t hidden, int64_t topk, int64_t moeExpertNum,
-                                            int64_t gmm1HLen, int64_t quantMode);
+                                            int64_t gmm1HLen, int64_t shareGmm1HLen, int64_t quantMode);
 
 /*
  * extension: softmax + top-k router. logits [T, E] fp32 -> topkIndex [T, K]

@@ -234,24 +234,31 @@ class Buffer:
                 self._ti(w), self._ti(dst), self.comm, capi.stream_ptr(), 0))
         return dst
 
-    def fused_workspace_bytes(self, tokens, hidden, topk, num_experts, gmm1_h_len, quant_mode):
-        n = self.lib.zbal_fused_deep_moe_workspace_size(tokens, hidden, topk, num_experts, gmm1_h_len, quant_mode)
+    def fused_workspace_bytes(self, tokens, hidden, topk, num_experts, gmm1_h_len, quant_mode, share_gmm1_h_len=0):
+        n = self.lib.zbal_fused_deep_moe_workspace_size(tokens, hidden, topk, num_experts, gmm1_h_len, share_gmm1_h_len,
+                                                        quant_mode)
         if n == 0:
             raise ValueError("invalid fused MoE shape")
         return int(n)
 
     def fused_deep_moe(self, x, topk_idx, gmm1_permuted_weight, gmm1_permuted_weight_scale, gmm2_weight,
                        gmm2_weight_scale, topk_weights, num_experts, quant_mode=0, expert_smooth_scales=None,
-                       workspace=None, out=None):
-        """zbal_deepep.cpp:658-802. Weights are pre-packed ([E,N,K]). Returns (output, expert_token_nums)."""
+                       share_gmm1_weight=None, share_gmm1_scale=None, share_gmm2_weight=None, share_gmm2_scale=None,
+                       share_smooth_scales=None, workspace=None, out=None):
+        """zbal_deepep.cpp:658-802. Weights are pre-packed (prepack_weight; shared-expert weights as [1,N,K]).
+        Returns (output, share_output, expert_token_nums) like the reference; share_output is None without a shared
+        expert."""
         T, H = x.shape
         K = topk_idx.shape[1]
         n1 = gmm1_permuted_weight.shape[1]
+        shared = share_gmm1_weight is not None
+        sn1 = share_gmm1_weight.shape[-2] if shared else 0
         expert_ids = topk_idx if topk_idx.dtype == torch.int32 else topk_idx.to(torch.int32)
         if workspace is None:
-            workspace = self._empty((self.fused_workspace_bytes(T, H, K, num_experts, n1, quant_mode),), torch.uint8)
+            workspace = self._empty((self.fused_workspace_bytes(T, H, K, num_experts, n1, quant_mode, sn1),), torch.uint8)
         if out is None:
             out = self._empty((T, H), x.dtype)
+        share_out = self._empty((T, H), x.dtype) if shared else None
         token_nums = self._empty((num_experts,), torch.int64)
         wdt = {0: None, 1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[quant_mode]
         null = ctypes.byref(capi.TensorInfo())
@@ -261,6 +268,11 @@ class Buffer:
             self._ti(gmm1_permuted_weight_scale),
             self._ti(gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), self._ti(gmm2_weight_scale),
             self._ti(topk_weights), self._ti(expert_smooth_scales) if expert_smooth_scales is not None else null,
-            null, null, null, null, null, null, self._ti(out), null, self._ti(token_nums), self._ti(workspace),
-            num_experts, quant_mode, 0, n1, 0, 0, self.comm, capi.stream_ptr(), 0))
-        return out, token_nums
+            self._ti(share_gmm1_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED) if shared else null,
+            self._ti(share_gmm1_scale) if shared else null,
+            self._ti(share_gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED) if shared else null,
+            self._ti(share_gmm2_scale) if shared else null,
+            self._ti(share_smooth_scales) if share_smooth_scales is not None else null,
+            null, self._ti(out), self._ti(share_out) if shared else null, self._ti(token_nums), self._ti(workspace),
+            num_experts, quant_mode, 0, n1, sn1, 0, self.comm, capi.stream_ptr(), 0))
+        return out, share_out, token_nums

@@ -97,7 +97,7 @@ SIGNATURES = {
                                          _TI, _TI, _vp, _vp, _i64]),
     "zbal_combine_low_latency": (_i32, [_TI, _TI, _TI, _TI, _TI, _TI, _i64, _vp, _vp, _i64]),
     "zbal_fused_deep_moe": (_i32, [_TI] * 18 + [_i64] * 6 + [_vp, _vp, _i64]),
-    "zbal_fused_deep_moe_workspace_size": (_u64, [_i64] * 6),
+    "zbal_fused_deep_moe_workspace_size": (_u64, [_i64] * 7),
     "zbal_moe_topk_route": (_i32, [_TI, _i64, _TI, _TI, _vp, _vp, _i64]),
     "zbal_moe_weight_prepack": (_i32, [_TI, _TI, _vp, _vp, _i64]),
     # zbal_hip_kernels.h
@@ -110,6 +110,7 @@ SIGNATURES = {
                                             _vp, _vp, _i32, _vp]),
     "zbalhip_reduce": (_i32, [ctypes.POINTER(_vp), _i32, _i64, _i32, _i32, _vp, _vp]),
     "zbalhip_weight_prepack": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp]),
+    "zbalhip_fill_i32": (_i32, [_vp, _i64, _i32, _vp]),
     "zbalhip_fused_permute_quant": (_i32, [_vp, _i32, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp,
                                            _vp, _i32, _vp]),
     "zbalhip_gmm1_swiglu_quant": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),

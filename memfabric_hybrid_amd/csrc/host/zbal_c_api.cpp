@@ -276,22 +276,24 @@ ZBAL_API int32_t zbal_fused_deep_moe(
     ZBAL_VALIDATE_RETURN(moeExpertNum > 0, "FusedDeepMoe failed as moeExpertNum " << moeExpertNum << " is invalid", Z_INVALID_PARAM);
     ZBAL_VALIDATE_RETURN(gmm1HLen > 0, "FusedDeepMoe failed as gmm1HLen " << gmm1HLen << " is invalid", Z_INVALID_PARAM);
     auto present = [](const zbal_tensor_info_t *t) { return t != nullptr && t->data != nullptr; };
-    ZBAL_VALIDATE_RETURN(!present(shareGmm1Weight) && !present(shareGmm1Scale) && !present(shareGmm2Weight) && !present(shareGmm2Scale) && !present(shareSmoothScales) && !present(shareOutput) && shareGmm1HLen == 0, "FusedDeepMoe failed as shared-expert operands are not supported", Z_INVALID_PARAM);
+    const bool shared = present(shareGmm1Weight);
+    ZBAL_VALIDATE_RETURN(shared == present(shareGmm1Scale) && shared == present(shareGmm2Weight) && shared == present(shareGmm2Scale) && shared == present(shareOutput) && shared == (shareGmm1HLen > 0) && (shared || !present(shareSmoothScales)), "FusedDeepMoe failed as the shared expert needs both weights, both scales, shareOutput and shareGmm1HLen > 0, or none of them", Z_INVALID_PARAM);
     ZBAL_VALIDATE_RETURN(isTensorList == 0, "FusedDeepMoe failed as tensor-list weights are not supported", Z_INVALID_PARAM);
     CommunicatorPtr c = Resolve("FusedDeepMoe", comm);
     if (!c) return Z_INVALID_PARAM;
     return c->FusedDeepMoe(x, expertIds, gmm1Weight, gmm1Scale, gmm2Weight, gmm2Scale, expertScales, expertSmoothScales,
-                           xActiveMask, output, expertTokenNums, workspace, moeExpertNum, quantMode, globalBs, gmm1HLen,
-                           stream, flags);
+                           shareGmm1Weight, shareGmm1Scale, shareGmm2Weight, shareGmm2Scale, shareSmoothScales, xActiveMask,
+                           output, shareOutput, expertTokenNums, workspace, moeExpertNum, quantMode, globalBs, gmm1HLen,
+                           shareGmm1HLen, stream, flags);
 }
 
 /* ---- extensions -------------------------------------------------------------------------- */
 
 ZBAL_API uint64_t zbal_fused_deep_moe_workspace_size(int64_t tokens, int64_t hidden, int64_t topk, int64_t moeExpertNum,
-                                                     int64_t gmm1HLen, int64_t quantMode)
+                                                     int64_t gmm1HLen, int64_t shareGmm1HLen, int64_t quantMode)
 {
     FusedWorkspace ws;
-    if (!PlanFusedWorkspace(tokens, hidden, topk, moeExpertNum, gmm1HLen, quantMode, &ws)) return 0;
+    if (!PlanFusedWorkspace(tokens, hidden, topk, moeExpertNum, gmm1HLen, shareGmm1HLen, quantMode, &ws)) return 0;
     return ws.total;
 }
 

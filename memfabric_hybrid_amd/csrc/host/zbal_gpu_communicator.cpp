@@ -17,6 +17,8 @@
 
 namespace zbal {
 
+static uint64_t Align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
+
 namespace {
 
 int64_t Numel(const zbal_tensor_info_t *t)
@@ -364,14 +366,56 @@ public:
                                             stream));
     }
 
+    /* shapes and types of one FFN's weights and scales: `experts` experts of [H, N1] and [N1/2, H] */
+    bool CheckFfnWeights(const char *op, const char *who, int mode, int64_t experts, int64_t H, int64_t N1,
+                         const zbal_tensor_info_t *w1, const zbal_tensor_info_t *s1, const zbal_tensor_info_t *w2,
+                         const zbal_tensor_info_t *s2, int *wscale2Dt)
+    {
+        const int64_t I = N1 / 2;
+        const int wdt = mode == 1 ? ZBAL_DATA_TYPE_INT8 : (mode == 2 ? ZBAL_DATA_TYPE_FP8_E4M3 : ZBAL_DATA_TYPE_INT4X2);
+        const int wdt_alt = mode == 2 ? ZBAL_DATA_TYPE_UINT8 : wdt;
+        const int64_t wdiv = mode == 3 ? 2 : 1;
+        ZBAL_VALIDATE_RETURN(N1 > 0 && N1 % 256 == 0, op << " failed as the " << who << " gmm1 width " << N1
+                                                         << " must be a positive multiple of 256", false);
+        ZBAL_VALIDATE_RETURN(w1->reserved[0] == ZBAL_WEIGHT_FORMAT_PREPACKED && w2->reserved[0] == ZBAL_WEIGHT_FORMAT_PREPACKED,
+                             op << " failed as the " << who << " weights are not pre-packed (zbal_moe_weight_prepack)", false);
+        auto check = [&](const char *name, const zbal_tensor_info_t *t, int dtA, int dtB, int64_t minElems) {
+            ZBAL_VALIDATE_RETURN(t->data != nullptr, op << " failed as " << who << " " << name << " has no data", false);
+            ZBAL_VALIDATE_RETURN(t->dataType == dtA || t->dataType == dtB,
+                                 op << " failed as " << who << " " << name << " has data type " << t->dataType, false);
+            ZBAL_VALIDATE_RETURN(Numel(t) >= minElems, op << " failed as " << who << " " << name << " holds " << Numel(t)
+                                                          << " elements, needs " << minElems, false);
+            return true;
+        };
+        if (!check("gmm1Weight", w1, wdt, wdt_alt, experts * H * N1 / wdiv)) return false;
+        if (!check("gmm2Weight", w2, wdt, wdt_alt, experts * I * H / wdiv)) return false;
+        *wscale2Dt = ZBAL_DATA_TYPE_FP32;
+        if (mode == 1) {
+            if (!check("gmm1Scale", s1, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, experts * N1)) return false;
+            if (!check("gmm2Scale", s2, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP32, experts * H)) return false;
+            *wscale2Dt = s2->dataType;
+        } else if (mode == 2) {
+            if (!check("gmm1Scale", s1, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, experts * (H / 128) * (N1 / 128))) return false;
+            if (!check("gmm2Scale", s2, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, experts * (I / 128) * (H / 128))) return false;
+        } else {
+            if (!check("gmm1Scale", s1, ZBAL_DATA_TYPE_FP16, ZBAL_DATA_TYPE_FP16, experts * (H / 128) * N1)) return false;
+            if (!check("gmm2Scale", s2, ZBAL_DATA_TYPE_FP16, ZBAL_DATA_TYPE_FP16, experts * (I / 128) * H)) return false;
+            *wscale2Dt = ZBAL_DATA_TYPE_FP16;
+        }
+        return true;
+    }
+
     int32_t FusedDeepMoe(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds,
                          const zbal_tensor_info_t *gmm1Weight, const zbal_tensor_info_t *gmm1Scale,
                          const zbal_tensor_info_t *gmm2Weight, const zbal_tensor_info_t *gmm2Scale,
                          const zbal_tensor_info_t *expertScales, const zbal_tensor_info_t *expertSmoothScales,
-                         const zbal_tensor_info_t *xActiveMask, const zbal_tensor_info_t *output,
+                         const zbal_tensor_info_t *shareGmm1Weight, const zbal_tensor_info_t *shareGmm1Scale,
+                         const zbal_tensor_info_t *shareGmm2Weight, const zbal_tensor_info_t *shareGmm2Scale,
+                         const zbal_tensor_info_t *shareSmoothScales, const zbal_tensor_info_t *xActiveMask,
+                         const zbal_tensor_info_t *output, const zbal_tensor_info_t *shareOutput,
                          const zbal_tensor_info_t *expertTokenNums, const zbal_tensor_info_t *workspace,
-                         int64_t moeExpertNum, int64_t quantMode, int64_t, int64_t gmm1HLen, aclrtStream stream,
-                         int64_t) override
+                         int64_t moeExpertNum, int64_t quantMode, int64_t, int64_t gmm1HLen, int64_t shareGmm1HLen,
+                         aclrtStream stream, int64_t) override
     {
         const char *op = "FusedDeepMoe";
         if (!SingleRank(op)) return Z_INVALID_PARAM;
@@ -385,45 +429,38 @@ public:
         ZBAL_VALIDATE_RETURN(expertIds->dim == 2 && expertIds->shape[0] == T, op << " failed as expertIds must be [tokens, topk]",
                              Z_INVALID_PARAM);
         const int64_t K = expertIds->shape[1], E = moeExpertNum, N1 = gmm1HLen, I = N1 / 2;
+        const bool shared = shareGmm1Weight != nullptr && shareGmm1Weight->data != nullptr;
+        const int64_t SN1 = shared ? shareGmm1HLen : 0, SI = SN1 / 2;
         ZBAL_VALIDATE_RETURN(K <= 32, op << " failed as topk " << K << " exceeds 32", Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(E <= 1024, op << " failed as moeExpertNum exceeds 1024", Z_INVALID_PARAM);
-        ZBAL_VALIDATE_RETURN(N1 % 256 == 0 && H % 256 == 0,
-                             op << " failed as gmm1HLen " << N1 << " and hidden " << H << " must be multiples of 256",
-                             Z_INVALID_PARAM);
-        ZBAL_VALIDATE_RETURN(gmm1Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_PREPACKED &&
-                                 gmm2Weight->reserved[0] == ZBAL_WEIGHT_FORMAT_PREPACKED,
-                             op << " failed as the weights are not pre-packed (zbal_moe_weight_prepack)", Z_INVALID_PARAM);
-        const int wdt = mode == 1 ? ZBAL_DATA_TYPE_INT8 : (mode == 2 ? ZBAL_DATA_TYPE_FP8_E4M3 : ZBAL_DATA_TYPE_INT4X2);
-        const int wdt_alt = mode == 2 ? ZBAL_DATA_TYPE_UINT8 : wdt;
-        const int64_t wdiv = mode == 3 ? 2 : 1;
+        ZBAL_VALIDATE_RETURN(H % 256 == 0, op << " failed as hidden " << H << " must be a multiple of 256", Z_INVALID_PARAM);
         ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
         ZB_CHECK(op, "output", output, x->dataType, x->dataType, T * H);
         ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
         ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
-        ZB_CHECK(op, "gmm1Weight", gmm1Weight, wdt, wdt_alt, E * H * N1 / wdiv);
-        ZB_CHECK(op, "gmm2Weight", gmm2Weight, wdt, wdt_alt, E * I * H / wdiv);
         ZB_CHECK(op, "expertTokenNums", expertTokenNums, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
-        int wscale2Dt = ZBAL_DATA_TYPE_FP32;
-        if (mode == 1) {
-            ZB_CHECK(op, "gmm1Scale", gmm1Scale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * N1);
-            ZB_CHECK(op, "gmm2Scale", gmm2Scale, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP32, E * H);
-            wscale2Dt = gmm2Scale->dataType;
-        } else if (mode == 2) {
-            ZB_CHECK(op, "gmm1Scale", gmm1Scale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * (H / 128) * (N1 / 128));
-            ZB_CHECK(op, "gmm2Scale", gmm2Scale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * (I / 128) * (H / 128));
-        } else {
-            ZB_CHECK(op, "gmm1Scale", gmm1Scale, ZBAL_DATA_TYPE_FP16, ZBAL_DATA_TYPE_FP16, E * (H / 128) * N1);
-            ZB_CHECK(op, "gmm2Scale", gmm2Scale, ZBAL_DATA_TYPE_FP16, ZBAL_DATA_TYPE_FP16, E * (I / 128) * H);
-            wscale2Dt = ZBAL_DATA_TYPE_FP16;
-        }
-        const float *smooth = nullptr;
+        int wscale2Dt = ZBAL_DATA_TYPE_FP32, shareWscale2Dt = ZBAL_DATA_TYPE_FP32;
+        if (!CheckFfnWeights(op, "expert", mode, E, H, N1, gmm1Weight, gmm1Scale, gmm2Weight, gmm2Scale, &wscale2Dt))
+            return Z_INVALID_PARAM;
+        const float *smooth = nullptr, *shareSmooth = nullptr;
         if (expertSmoothScales && expertSmoothScales->data) {
             ZBAL_VALIDATE_RETURN(mode != 2, op << " failed as smooth scales do not apply to the fp8 mode", Z_INVALID_PARAM);
             ZB_CHECK(op, "expertSmoothScales", expertSmoothScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, E * H);
             smooth = (const float *)expertSmoothScales->data;
         }
+        if (shared) {
+            if (!CheckFfnWeights(op, "shared", mode, 1, H, SN1, shareGmm1Weight, shareGmm1Scale, shareGmm2Weight,
+                                 shareGmm2Scale, &shareWscale2Dt))
+                return Z_INVALID_PARAM;
+            ZB_CHECK(op, "shareOutput", shareOutput, x->dataType, x->dataType, T * H);
+            if (shareSmoothScales && shareSmoothScales->data) {
+                ZBAL_VALIDATE_RETURN(mode != 2, op << " failed as smooth scales do not apply to the fp8 mode", Z_INVALID_PARAM);
+                ZB_CHECK(op, "shareSmoothScales", shareSmoothScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, H);
+                shareSmooth = (const float *)shareSmoothScales->data;
+            }
+        }
         FusedWorkspace ws;
-        ZBAL_VALIDATE_RETURN(PlanFusedWorkspace(T, H, K, E, N1, quantMode, &ws), op << " failed as the shapes are invalid",
+        ZBAL_VALIDATE_RETURN(PlanFusedWorkspace(T, H, K, E, N1, SN1, quantMode, &ws), op << " failed as the shapes are invalid",
                              Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(workspace->data != nullptr && (reinterpret_cast<uintptr_t>(workspace->data) & 255u) == 0,
                              op << " failed as the workspace is null or not 256-byte aligned", Z_INVALID_PARAM);
@@ -443,15 +480,38 @@ public:
         float *scale2 = (float *)(base + ws.scale2);
         float *sgl = mode == 2 ? nullptr : (float *)(base + ws.sgl);
         void *y = base + ws.y;
+        const int qmode = mode == 2 ? 2 : 1;
         if (T == 0) { /* nothing routed: counts are zero */
             return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, 0,
-                                                            H, K, E, mode == 2 ? 2 : 1, q1, xs, expandIdx,
+                                                            H, K, E, qmode, q1, xs, expandIdx,
                                                             (int64_t *)expertTokenNums->data, rowOff, scratch,
                                                             ZBALHIP_LAYOUT_MAX_BLOCKS, stream));
         }
-        int32_t rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, T, H, K, E,
-                                                 mode == 2 ? 2 : 1, q1, xs, expandIdx, (int64_t *)expertTokenNums->data,
-                                                 rowOff, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
+        int32_t rc = 0;
+        if (shared) {
+            /*
+             * The shared expert is the same pipeline with one expert that every token picks once: the rows stay in
+             * token order, so the second GEMM writes shareOutput directly. It runs first and borrows the routed
+             * pass's workspace regions (sized for the larger of the two); its all-zero expert ids and its one count
+             * sit at the start of the y region, which nothing else uses until the routed second GEMM.
+             */
+            int32_t *zeroIds = (int32_t *)y;
+            int64_t *shareCount = (int64_t *)((uint8_t *)y + Align256((uint64_t)T * 4));
+            rc = zbalhip_fill_i32(zeroIds, T, 0, stream);
+            if (rc != 0) return Launched(op, rc);
+            rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, T, H, 1, 1, qmode, q1, xs, expandIdx,
+                                             shareCount, rowOff, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
+            if (rc != 0) return Launched(op, rc);
+            rc = zbalhip_gmm1_swiglu_quant(q1, xs, shareGmm1Weight->data, shareGmm1Scale->data, rowOff, 1, T, H, SN1, mode,
+                                           q2, scale2, sgl, stream);
+            if (rc != 0) return Launched(op, rc);
+            rc = zbalhip_gmm2_dequant(q2, scale2, shareGmm2Weight->data, shareGmm2Scale->data, shareWscale2Dt, rowOff, 1, T,
+                                      SI, H, mode, x->dataType, shareOutput->data, stream);
+            if (rc != 0) return Launched(op, rc);
+        }
+        rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, T, H, K, E, qmode, q1,
+                                         xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff, scratch,
+                                         ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
         if (rc != 0) return Launched(op, rc);
         rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1, mode, q2, scale2,
                                        sgl, stream);
@@ -500,16 +560,19 @@ public:
 
 CommunicatorPtr MakeGpuCommunicator(const GroupInfo &info) { return std::make_shared<GpuCommunicator>(info); }
 
-static uint64_t Align256(uint64_t v) { return (v + 255u) & ~uint64_t(255); }
 
-bool PlanFusedWorkspace(int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int64_t n1, int64_t quantMode,
-                        FusedWorkspace *ws)
+bool PlanFusedWorkspace(int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int64_t n1, int64_t shareN1,
+                        int64_t quantMode, FusedWorkspace *ws)
 {
-    if (tokens < 0 || hidden <= 0 || topk <= 0 || experts <= 0 || n1 <= 0 || quantMode < 0 || quantMode > 3) return false;
-    if (hidden % 128 != 0 || n1 % 256 != 0) return false;
+    if (tokens < 0 || hidden <= 0 || topk <= 0 || experts <= 0 || n1 <= 0 || shareN1 < 0 || quantMode < 0 || quantMode > 3)
+        return false;
+    if (hidden % 128 != 0 || n1 % 256 != 0 || shareN1 % 256 != 0) return false;
     const uint64_t rows = (uint64_t)(tokens * topk > 0 ? tokens * topk : 1);
-    const uint64_t H = hidden, I = n1 / 2, E = experts;
+    const uint64_t T = (uint64_t)(tokens > 0 ? tokens : 1);
+    const uint64_t H = hidden, I = n1 / 2, SI = shareN1 / 2, E = experts;
     const bool fp8 = quantMode == 2;
+    /* the shared expert's pass (T rows, width SI) reuses the regions of the routed pass (rows rows, width I) */
+    auto both = [&](uint64_t routed, uint64_t shared) { return SI > 0 && shared > routed ? shared : routed; };
     uint64_t off = 0;
     auto take = [&](uint64_t bytes) { uint64_t o = off; off = Align256(off + bytes); return o; };
     ws->q1 = take(rows * H);
@@ -518,10 +581,10 @@ bool PlanFusedWorkspace(int64_t tokens, int64_t hidden, int64_t topk, int64_t ex
     ws->counts = take(E * 8);
     ws->row_off = take((E + 1) * 4);
     ws->layout_scratch = take((uint64_t)ZBALHIP_LAYOUT_MAX_BLOCKS * E * 4);
-    ws->q2 = take(rows * I);
-    ws->scale2 = take(rows * (fp8 ? (I + 127) / 128 : 1) * 4);
-    ws->sgl = fp8 ? off : take(rows * (I + 1) * 4);
-    ws->y = take(rows * H * 2);
+    ws->q2 = take(both(rows * I, T * SI));
+    ws->scale2 = take(both(rows * (fp8 ? (I + 127) / 128 : 1), T * (fp8 ? (SI + 127) / 128 : 1)) * 4);
+    ws->sgl = fp8 ? off : take(both(rows * (I + 1), T * (SI + 1)) * 4);
+    ws->y = take(both(rows * H * 2, Align256(T * 4) + 256));
     ws->total = off;
     return true;
 }

@@ -163,10 +163,13 @@ public:
                                  const zbal_tensor_info_t *gmm1Weight, const zbal_tensor_info_t *gmm1Scale,
                                  const zbal_tensor_info_t *gmm2Weight, const zbal_tensor_info_t *gmm2Scale,
                                  const zbal_tensor_info_t *expertScales, const zbal_tensor_info_t *expertSmoothScales,
-                                 const zbal_tensor_info_t *xActiveMask, const zbal_tensor_info_t *output,
+                                 const zbal_tensor_info_t *shareGmm1Weight, const zbal_tensor_info_t *shareGmm1Scale,
+                                 const zbal_tensor_info_t *shareGmm2Weight, const zbal_tensor_info_t *shareGmm2Scale,
+                                 const zbal_tensor_info_t *shareSmoothScales, const zbal_tensor_info_t *xActiveMask,
+                                 const zbal_tensor_info_t *output, const zbal_tensor_info_t *shareOutput,
                                  const zbal_tensor_info_t *expertTokenNums, const zbal_tensor_info_t *workspace,
                                  int64_t moeExpertNum, int64_t quantMode, int64_t globalBs, int64_t gmm1HLen,
-                                 aclrtStream stream, int64_t flags) = 0;
+                                 int64_t shareGmm1HLen, aclrtStream stream, int64_t flags) = 0;
     virtual int32_t TopkRoute(const zbal_tensor_info_t *logits, int64_t topkNum, const zbal_tensor_info_t *topkIndex,
                               const zbal_tensor_info_t *topkWeight, aclrtStream stream, int64_t flags) = 0;
     virtual int32_t WeightPrepack(const zbal_tensor_info_t *src, const zbal_tensor_info_t *dst, aclrtStream stream,
@@ -198,8 +201,9 @@ uint32_t Count();
 struct FusedWorkspace {
     uint64_t q1, xs, expand_idx, counts, row_off, layout_scratch, q2, scale2, sgl, y, total;
 };
-bool PlanFusedWorkspace(int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int64_t n1, int64_t quantMode,
-                        FusedWorkspace *ws);
+/* shareN1 = output width of the shared expert's first GEMM, 0 without a shared expert */
+bool PlanFusedWorkspace(int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int64_t n1, int64_t shareN1,
+                        int64_t quantMode, FusedWorkspace *ws);
 
 } // namespace zbal
 

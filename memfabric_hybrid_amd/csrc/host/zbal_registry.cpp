@@ -53,8 +53,10 @@ public:
     int32_t FusedDeepMoe(const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                          const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                          const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
+                         const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
+                         const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                          const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *, int64_t,
-                         int64_t, int64_t, int64_t, aclrtStream, int64_t) override { return Z_OK; }
+                         int64_t, int64_t, int64_t, int64_t, aclrtStream, int64_t) override { return Z_OK; }
     int32_t TopkRoute(const zbal_tensor_info_t *, int64_t, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                       aclrtStream, int64_t) override { return Z_OK; }
     int32_t WeightPrepack(const zbal_tensor_info_t *, const zbal_tensor_info_t *, aclrtStream, int64_t) override { return Z_OK; }

@@ -328,6 +328,11 @@ topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int
     }
 }
 
+__global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v)
+{
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
+}
+
 inline int ceil_log2(int64_t v)
 {
     int b = 0;
@@ -391,6 +396,16 @@ static bool layout_args_ok(int64_t tokens, int64_t experts, int64_t topk)
 {
     return tokens >= 0 && tokens <= 0x7fffffff / (topk > 0 ? topk : 1) && experts > 0 && experts <= ZB_MAX_EXPERTS &&
            topk > 0;
+}
+
+extern "C" int32_t zbalhip_fill_i32(int32_t *p, int64_t n, int32_t value, void *stream)
+{
+    if (n < 0 || (n > 0 && !p)) return ZBALHIP_INVALID;
+    if (n == 0) return ZBALHIP_OK;
+    int64_t blocks = (n + 255) / 256;
+    if (blocks > 1024) blocks = 1024;
+    fill_i32_kernel<<<(unsigned)blocks, 256, 0, (hipStream_t)stream>>>(p, n, value);
+    return zbalhip_check_launch();
 }
 
 extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64_t experts, int64_t topk,

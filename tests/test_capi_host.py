@@ -184,6 +184,8 @@ def test_operator_validation_codes(host_world):
     assert lib.zbal_fused_deep_moe(*fused, 0, 0, 0, 256, 0, 0, world, None, 0) == -2
     assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 0, 0, 0, world, None, 0) == -2
     assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 256, 0, 1, world, None, 0) == -2              # tensor list
+    half = list(fused); half[8] = ctypes.byref(capi.TensorInfo(data=ctypes.c_void_p(0x1000)))  # shared gmm1 weight alone
+    assert lib.zbal_fused_deep_moe(*half, 8, 0, 0, 256, 256, 0, world, None, 0) == -2
     bad = list(fused); bad[17] = None
     assert lib.zbal_fused_deep_moe(*bad, 8, 0, 0, 256, 0, 0, world, None, 0) == -2                # workspace
     assert lib.zbal_comm_register_peer_window(world, 9, p, 64) == -2
@@ -193,9 +195,13 @@ def test_operator_validation_codes(host_world):
 
 def test_fused_workspace_size_is_monotonic(lib):
     f = lib.zbal_fused_deep_moe_workspace_size
-    assert f(0, 7168, 8, 32, 4096, 2) > 0
-    a, b = f(128, 7168, 8, 32, 4096, 0), f(256, 7168, 8, 32, 4096, 0)
+    assert f(0, 7168, 8, 32, 4096, 0, 2) > 0
+    a, b = f(128, 7168, 8, 32, 4096, 0, 0), f(256, 7168, 8, 32, 4096, 0, 0)
     assert 0 < a < b
-    assert f(128, 7168, 8, 32, 4000, 0) == 0 and f(128, 100, 8, 32, 4096, 0) == 0 and f(128, 7168, 8, 32, 4096, 9) == 0
+    assert f(128, 7168, 8, 32, 4000, 0, 0) == 0 and f(128, 100, 8, 32, 4096, 0, 0) == 0 and f(128, 7168, 8, 32, 4096, 0, 9) == 0
     # W8A8 keeps an fp32 SwiGLU scratch that the fp8 mode does not need
-    assert f(128, 7168, 8, 32, 4096, 2) < f(128, 7168, 8, 32, 4096, 0)
+    assert f(128, 7168, 8, 32, 4096, 0, 2) < f(128, 7168, 8, 32, 4096, 0, 0)
+    # a shared expert reuses the routed pass's regions: only one wider than topk routed experts adds bytes
+    assert f(128, 7168, 8, 32, 4096, 4096, 0) == a
+    assert f(128, 7168, 1, 32, 512, 4096, 0) > f(128, 7168, 1, 32, 512, 0, 0)
+    assert f(128, 7168, 8, 32, 4096, 100, 0) == 0

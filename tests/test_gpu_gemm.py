@@ -232,7 +232,7 @@ def run_fused(buf, x, ids, es, w1, s1, w2, s2, E, mode, smooth=None, xdt=torch.b
     w2p = buf.prepack_weight(dev(w2), int4=int4)
     sdt1 = torch.float16 if mode == 3 else None
     sdt2 = torch.float16 if mode == 3 else torch.bfloat16
-    out, nums = buf.fused_deep_moe(dev(x, xdt), dev(ids), w1p, dev(s1, sdt1), w2p, dev(s2, sdt2), dev(es), E,
+    out, _, nums = buf.fused_deep_moe(dev(x, xdt), dev(ids), w1p, dev(s1, sdt1), w2p, dev(s2, sdt2), dev(es), E,
                                    quant_mode=mode, expert_smooth_scales=dev(smooth) if smooth is not None else None)
     return host(out), host(nums)
 
@@ -293,7 +293,7 @@ def test_prefill_share_full_size_sampled_tokens(buf):
         return w, sc
     w1, s1 = weights(H, 2 * I)
     w2, s2 = weights(I, H)
-    out, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1), s1, buf.prepack_weight(w2), s2, es, E, quant_mode=2)
+    out, _, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1), s1, buf.prepack_weight(w2), s2, es, E, quant_mode=2)
     torch.cuda.synchronize()
     ids_h = host(ids)
     assert np.array_equal(host(nums), np.bincount(ids_h.ravel(), minlength=E))
@@ -331,7 +331,7 @@ def test_decode_share_full_size_bit_exact(buf):
     w1, s1 = _int_weights(g, 1, E, H, 2 * I)
     w2, s2 = _int_weights(g, 1, E, I, H)
     s2 = s2.to(torch.bfloat16)
-    out, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1), s1, buf.prepack_weight(w2), s2, es, E, quant_mode=1)
+    out, _, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1), s1, buf.prepack_weight(w2), s2, es, E, quant_mode=1)
     ref, counts = zo.fused_moe(_bits16(x), zo.DT_BF16, host(ids), host(es), host(w1), host(s1), host(w2), _bits16(s2), E, 1)
     assert np.array_equal(host(nums), counts)
     assert np.array_equal(_bits16(out), ref)
@@ -346,7 +346,7 @@ def test_w4a8_layer_full_size_sampled_tokens_bit_exact(buf):
     ids, es = buf.topk_route(torch.rand((T, E), device="cuda", generator=g), K)
     w1, s1 = _int_weights(g, 3, E, H, 2 * I)
     w2, s2 = _int_weights(g, 3, E, I, H)
-    out, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1, int4=True), s1, buf.prepack_weight(w2, int4=True), s2, es, E,
+    out, _, nums = buf.fused_deep_moe(x, ids, buf.prepack_weight(w1, int4=True), s1, buf.prepack_weight(w2, int4=True), s2, es, E,
                                    quant_mode=3)
     ids_h = host(ids)
     assert np.array_equal(host(nums), np.bincount(ids_h.ravel(), minlength=E))
@@ -354,6 +354,38 @@ def test_w4a8_layer_full_size_sampled_tokens_bit_exact(buf):
     ref, _ = zo.fused_moe(_bits16(x)[pick], zo.DT_BF16, ids_h[pick], host(es)[pick], host(w1), _bits16(s1), host(w2), _bits16(s2),
                           E, 3)
     assert np.array_equal(_bits16(out)[pick], ref)
+
+
+@pytest.mark.parametrize("mode", [0, 2, 3])
+@pytest.mark.parametrize("share_i,smooth", [(128, False), (640, True)])
+def test_fused_moe_shared_expert(buf, mode, share_i, smooth):
+    """The shared expert (zbal_kernel_fused_deep_moe.h:470-472): one more expert, applied to every token, whose result
+    goes to its own output. The oracle runs it as a one-expert layer in which every token picks expert 0 with weight 1
+    (multiplying by 1.0 and adding to 0 changes no bit). The routed output must not change."""
+    T, H, K, E, I = 70, 256, 4, 8, 128
+    if mode == 2 and smooth:
+        pytest.skip("smooth scales do not apply to the fp8 mode")
+    x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 90 + mode)
+    _, _, _, sw1, ss1, sw2, ss2 = fused_inputs(T, H, 1, 1, share_i, mode, 95 + mode)
+    ssm = rng(97).uniform(0.2, 1.0, (1, H)).astype(np.float32) if smooth else None
+    int4 = mode == 3
+    sdt1 = torch.float16 if mode == 3 else None
+    sdt2 = {0: torch.bfloat16, 1: torch.bfloat16, 2: None, 3: torch.float16}[mode]
+    pack = lambda w: buf.prepack_weight(dev(w), int4=int4)
+    out, share, nums = buf.fused_deep_moe(
+        dev(x, torch.bfloat16), dev(ids), pack(w1), dev(s1, sdt1), pack(w2), dev(s2, sdt2), dev(es), E, quant_mode=mode,
+        share_gmm1_weight=pack(sw1), share_gmm1_scale=dev(ss1, sdt1), share_gmm2_weight=pack(sw2),
+        share_gmm2_scale=dev(ss2, sdt2), share_smooth_scales=dev(ssm[0]) if smooth else None)
+    ref, counts = zo.fused_moe(x, zo.DT_BF16, ids, es, w1, s1, w2, s2, E, mode)
+    ref_share, _ = zo.fused_moe(x, zo.DT_BF16, np.zeros((T, 1), np.int64), np.ones((T, 1), np.float32), sw1, ss1, sw2, ss2, 1,
+                                mode, smooth=ssm)
+    assert np.array_equal(host(nums), counts)
+    if mode == 2:
+        assert max_rel_err(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(ref)) < 2e-2
+        assert max_rel_err(zo.bf16_to_f32(host(share)), zo.bf16_to_f32(ref_share)) < 2e-2
+    else:
+        assert np.array_equal(host(out), ref)
+        assert np.array_equal(host(share), ref_share)
 
 
 def test_fused_moe_empty_experts_and_invalid_ids(buf):
