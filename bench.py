@@ -186,7 +186,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
         capi.check("route", lib.zbalhip_topk_route(logits.data_ptr(), T, E, K, topk_idx.data_ptr(), topk_w.data_ptr(), st))
         ids32.copy_(topk_idx)
         evs[1].record()
-        capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, T, H, K, E,
+        capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, None, T, H, K, E,
                                                               2 if mode == 2 else 1, q1, xs, eidx, nums.data_ptr(), row_off,
                                                               scratch, 50, st))
         evs[2].record()

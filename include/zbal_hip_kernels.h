@@ -70,7 +70,8 @@ ZBALHIP_API int32_t zbalhip_dispatch_normal(const void *x, int32_t x_dtype, cons
 /*
  * Replaces ZBALOpCombineNormal (zbal_npu_operators.h:64-68; kernel
  * combine_normal.h:398-494): out[t] = round(sum_k fp32(y[base[e]+idx]) * w),
- * multiply and add rounded separately, k ascending, invalid ids skipped.
+ * multiply and add rounded separately, k ascending, invalid ids skipped; a
+ * token with a valid id but send_token_idx < 0 is not written at all.
  * base_is_inclusive = 1 reads `base` as the low-latency kernels' inclusive
  * running counts (combine_low_latency.h:504-506).
  */
@@ -126,9 +127,14 @@ ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int
  * fp32 multiplied in first; mode 2: e4m3 1x128. Outputs q1 [rows,H], xs
  * ([rows] or [rows,H/128]), expand_idx [T,K], counts [E] i64 and the
  * exclusive row offsets row_off [E+1] i32. scratch / scratch_blocks as above
- * (not touched).
+ * (not touched). active_mask (optional, one byte per token): only the first
+ * sum(mask) tokens are routed, as in the reference's TokenActiveMaskCal
+ * (…swiglu_quant_multistage_workspace.h:836-863); the picks of the others get
+ * expand_idx = -1, which zbalhip_combine reads as "leave this token's output
+ * row alone".
  */
 ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids, const float *smooth,
+                                    const uint8_t *active_mask,
                                     int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int32_t mode,
                                     void *q1, float *xs, int32_t *expand_idx, int64_t *counts, int32_t *row_off,
                                     int32_t *scratch, int32_t scratch_blocks, void *stream);

@@ -108,7 +108,9 @@ int32_t zbal_combine_low_latency(const zbal_tensor_info_t *expandX, const zbal_t
  * [shareGmm1HLen/2, H] pre-packed like the others, scales shaped as one
  * expert's, optional shareSmoothScales [H]; its result goes to shareOutput
  * [tokens, H] and is not added to output. Pass all of them or none.
- * xActiveMask and isTensorList != 0 are rejected with -2.
+ * xActiveMask [tokens] (one byte per token): only the first sum(mask)
+ * tokens are routed and written, as in the reference. isTensorList != 0 is
+ * rejected with -2.
  */
 int32_t zbal_fused_deep_moe(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds,
                             const zbal_tensor_info_t *gmm1Weight, const zbal_tensor_info_t *gmm1Scale,

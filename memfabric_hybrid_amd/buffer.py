@@ -244,10 +244,11 @@ class Buffer:
     def fused_deep_moe(self, x, topk_idx, gmm1_permuted_weight, gmm1_permuted_weight_scale, gmm2_weight,
                        gmm2_weight_scale, topk_weights, num_experts, quant_mode=0, expert_smooth_scales=None,
                        share_gmm1_weight=None, share_gmm1_scale=None, share_gmm2_weight=None, share_gmm2_scale=None,
-                       share_smooth_scales=None, workspace=None, out=None):
+                       share_smooth_scales=None, x_active_mask=None, workspace=None, out=None):
         """zbal_deepep.cpp:658-802. Weights are pre-packed (prepack_weight; shared-expert weights as [1,N,K]).
         Returns (output, share_output, expert_token_nums) like the reference; share_output is None without a shared
-        expert."""
+        expert. x_active_mask [T] bool: only the first sum(mask) tokens are routed; the other rows of `out` keep
+        their contents."""
         T, H = x.shape
         K = topk_idx.shape[1]
         n1 = gmm1_permuted_weight.shape[1]
@@ -273,6 +274,7 @@ class Buffer:
             self._ti(share_gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED) if shared else null,
             self._ti(share_gmm2_scale) if shared else null,
             self._ti(share_smooth_scales) if share_smooth_scales is not None else null,
-            null, self._ti(out), self._ti(share_out) if shared else null, self._ti(token_nums), self._ti(workspace),
+            self._ti(x_active_mask.view(torch.uint8)) if x_active_mask is not None else null,
+            self._ti(out), self._ti(share_out) if shared else null, self._ti(token_nums), self._ti(workspace),
             num_experts, quant_mode, 0, n1, sn1, 0, self.comm, capi.stream_ptr(), 0))
         return out, share_out, token_nums

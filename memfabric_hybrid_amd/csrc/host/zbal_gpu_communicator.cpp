@@ -419,8 +419,6 @@ public:
     {
         const char *op = "FusedDeepMoe";
         if (!SingleRank(op)) return Z_INVALID_PARAM;
-        ZBAL_VALIDATE_RETURN(xActiveMask == nullptr || xActiveMask->data == nullptr,
-                             op << " failed as xActiveMask is not supported", Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(quantMode >= 0 && quantMode <= 3, op << " failed as quantMode " << quantMode << " is invalid",
                              Z_INVALID_PARAM);
         const int mode = quantMode <= 1 ? 1 : (int)quantMode; /* 0 and 1 both mean W8A8, as in the reference kernel */
@@ -459,6 +457,11 @@ public:
                 shareSmooth = (const float *)shareSmoothScales->data;
             }
         }
+        const uint8_t *activeMask = nullptr;
+        if (xActiveMask && xActiveMask->data) { /* one bool per token; the first sum(mask) tokens are routed */
+            ZB_CHECK(op, "xActiveMask", xActiveMask, ZBAL_DATA_TYPE_UINT8, ZBAL_DATA_TYPE_INT8, T);
+            activeMask = (const uint8_t *)xActiveMask->data;
+        }
         FusedWorkspace ws;
         ZBAL_VALIDATE_RETURN(PlanFusedWorkspace(T, H, K, E, N1, SN1, quantMode, &ws), op << " failed as the shapes are invalid",
                              Z_INVALID_PARAM);
@@ -482,8 +485,8 @@ public:
         void *y = base + ws.y;
         const int qmode = mode == 2 ? 2 : 1;
         if (T == 0) { /* nothing routed: counts are zero */
-            return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, 0,
-                                                            H, K, E, qmode, q1, xs, expandIdx,
+            return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth,
+                                                            nullptr, 0, H, K, E, qmode, q1, xs, expandIdx,
                                                             (int64_t *)expertTokenNums->data, rowOff, scratch,
                                                             ZBALHIP_LAYOUT_MAX_BLOCKS, stream));
         }
@@ -499,7 +502,7 @@ public:
             int64_t *shareCount = (int64_t *)((uint8_t *)y + Align256((uint64_t)T * 4));
             rc = zbalhip_fill_i32(zeroIds, T, 0, stream);
             if (rc != 0) return Launched(op, rc);
-            rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, T, H, 1, 1, qmode, q1, xs, expandIdx,
+            rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, nullptr, T, H, 1, 1, qmode, q1, xs, expandIdx,
                                              shareCount, rowOff, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
             if (rc != 0) return Launched(op, rc);
             rc = zbalhip_gmm1_swiglu_quant(q1, xs, shareGmm1Weight->data, shareGmm1Scale->data, rowOff, 1, T, H, SN1, mode,
@@ -509,8 +512,8 @@ public:
                                       SI, H, mode, x->dataType, shareOutput->data, stream);
             if (rc != 0) return Launched(op, rc);
         }
-        rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, T, H, K, E, qmode, q1,
-                                         xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff, scratch,
+        rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, activeMask, T, H, K, E,
+                                         qmode, q1, xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff, scratch,
                                          ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
         if (rc != 0) return Launched(op, rc);
         rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1, mode, q2, scale2,

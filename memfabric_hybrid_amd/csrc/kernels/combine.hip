@@ -29,13 +29,18 @@ combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base,
     __shared__ int s_n;
     const int t = blockIdx.x;
     if (threadIdx.x == 0) {
-        /* compact the valid picks, keeping their order */
+        /*
+         * Compact the valid picks, keeping their order. A pick with a valid expert but a negative rank belongs to a
+         * token that the layout masked out (x_active_mask): such a token's output row is left as it is.
+         */
         int n = 0;
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
             if (e < 0 || e >= experts) continue;
+            const int32_t rk = rank_in_expert[(int64_t)t * topk + k];
+            if (rk < 0) { n = -1; break; }
             const int32_t b = base_inclusive ? (e == 0 ? 0 : base[e - 1]) : base[e];
-            s_row[n] = (int64_t)b + rank_in_expert[(int64_t)t * topk + k];
+            s_row[n] = (int64_t)b + rk;
             s_w[n] = w[(int64_t)t * topk + k];
             ++n;
         }
@@ -43,6 +48,7 @@ combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base,
     }
     __syncthreads();
     const int n = s_n;
+    if (n < 0) return;
     const int nchunk = hidden / 8;
     for (int c = threadIdx.x; c < nchunk; c += blockDim.x) {
         float acc[8];

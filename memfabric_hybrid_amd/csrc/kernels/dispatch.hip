@@ -13,8 +13,9 @@
 #include "zbal_hip_kernels.h"
 
 int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
-                                      int32_t token_nums_type, int32_t *send_token_idx, int32_t *incl_i32,
-                                      int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed, hipStream_t st);
+                                      int32_t token_nums_type, const uint8_t *active_mask, int32_t *send_token_idx,
+                                      int32_t *incl_i32, int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed,
+                                      hipStream_t st);
 
 namespace {
 
@@ -112,8 +113,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         const int nblk128 = hidden / 128;
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts) continue;
-            const int64_t row = pick_row(base, base_inclusive, e, rank_in_expert[(int64_t)t * topk + k]);
+            const int rk = rank_in_expert[(int64_t)t * topk + k];
+            if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
+            const int64_t row = pick_row(base, base_inclusive, e, rk);
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
                 const int seg = s * blockDim.x + threadIdx.x;
@@ -141,8 +143,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         for (int s = 0; s < SLOTS; ++s) q[s] = pack16_i8(v[s], sq);
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts) continue;
-            const int64_t row = pick_row(base, base_inclusive, e, rank_in_expert[(int64_t)t * topk + k]);
+            const int rk = rank_in_expert[(int64_t)t * topk + k];
+            if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
+            const int64_t row = pick_row(base, base_inclusive, e, rk);
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
                 const int seg = s * blockDim.x + threadIdx.x;
@@ -154,8 +157,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
     } else {
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts) continue; /* uniform across the block */
-            const int64_t row = pick_row(base, base_inclusive, e, rank_in_expert[(int64_t)t * topk + k]);
+            const int rk = rank_in_expert[(int64_t)t * topk + k];
+            if (e < 0 || e >= experts || rk < 0) continue; /* uniform across the block */
+            const int64_t row = pick_row(base, base_inclusive, e, rk);
             float sv[SLOTS][16];
             float amax = 0.0f;
 #pragma unroll
@@ -202,8 +206,9 @@ permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ 
         }
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts) continue;
-            const int64_t row = pick_row(base, base_inclusive, e, rank_in_expert[(int64_t)t * topk + k]);
+            const int rk = rank_in_expert[(int64_t)t * topk + k];
+            if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
+            const int64_t row = pick_row(base, base_inclusive, e, rk);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u * blockDim.x + threadIdx.x;
@@ -299,7 +304,7 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
         scratch_blocks < 1)
         return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
-    const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, token_nums_type, expand_idx,
+    const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, token_nums_type, nullptr, expand_idx,
                                                      ep_recv_counts, nullptr, nullptr, expert_token_nums, st);
     if (rc != ZBALHIP_OK) return rc;
     const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_NOEPS : QM_FP8);
@@ -308,7 +313,8 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
 }
 
 extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids,
-                                               const float *smooth, int64_t tokens, int64_t hidden, int64_t topk,
+                                               const float *smooth, const uint8_t *active_mask, int64_t tokens,
+                                               int64_t hidden, int64_t topk,
                                                int64_t experts, int32_t mode, void *q1, float *xs, int32_t *expand_idx,
                                                int64_t *counts, int32_t *row_off, int32_t *scratch,
                                                int32_t scratch_blocks, void *stream)
@@ -318,8 +324,8 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
         return ZBALHIP_INVALID;
     if (mode == 2 && smooth) return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
-    const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, 1, expand_idx, nullptr, row_off,
-                                                     counts, nullptr, st);
+    const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, 1, active_mask, expand_idx, nullptr,
+                                                     row_off, counts, nullptr, st);
     if (rc != ZBALHIP_OK) return rc;
     return zbalhip_permute_internal(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk,
                                     experts, mode == 2 ? QM_FP8 : QM_INT8_NOEPS, q1, xs, st);

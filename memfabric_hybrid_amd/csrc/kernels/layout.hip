@@ -156,17 +156,38 @@ layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
 template <typename IdxT>
 __global__ void __launch_bounds__(ZB_FUSED_THREADS)
 layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int experts, int tpb, int nbits,
-                    int token_nums_type, int32_t *__restrict__ send_token_idx, int32_t *__restrict__ incl_i32,
-                    int32_t *__restrict__ row_off /* [E+1] */, int64_t *__restrict__ counts_i64,
-                    int64_t *__restrict__ nums_typed)
+                    int token_nums_type, const uint8_t *__restrict__ active_mask, int32_t *__restrict__ send_token_idx,
+                    int32_t *__restrict__ incl_i32, int32_t *__restrict__ row_off /* [E+1] */,
+                    int64_t *__restrict__ counts_i64, int64_t *__restrict__ nums_typed)
 {
     __shared__ int32_t run[ZB_MAX_EXPERTS];
     __shared__ int32_t wsum[ZB_FUSED_THREADS / 64];
+    __shared__ int32_t s_active;
     for (int e = threadIdx.x; e < experts; e += blockDim.x) run[e] = 0;
+    if (threadIdx.x == 0) s_active = 0;
     __syncthreads();
-    const int tok0 = blockIdx.x * tpb;
+    /*
+     * x_active_mask (one bool per token): the reference processes the first sum(mask) tokens and nothing else
+     * (TokenActiveMaskCal, fused_deep_moe/gemm/kernel/...swiglu_quant_multistage_workspace.h:836-863). Picks of
+     * the other tokens get rank -1 here, which the permute and combine kernels take as "not there".
+     */
+    int active = tokens;
+    if (active_mask) {
+        int part = 0;
+        for (int t = threadIdx.x; t < tokens; t += blockDim.x) part += active_mask[t] != 0;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if ((threadIdx.x & 63) == 0 && part) atomicAdd(&s_active, part);
+        __syncthreads();
+        active = s_active;
+    }
+    int tok0 = blockIdx.x * tpb;
     int tok1 = tok0 + tpb;
     if (tok1 > tokens) tok1 = tokens;
+    for (int64_t i = (int64_t)(tok0 > active ? tok0 : active) * topk + threadIdx.x; i < (int64_t)tok1 * topk; i += blockDim.x)
+        send_token_idx[i] = -1;
+    if (tok0 > active) tok0 = active;
+    if (tok1 > active) tok1 = active;
     const int64_t p0 = (int64_t)tok0 * topk, p1 = (int64_t)tok1 * topk;
     constexpr int PER = 16 / (int)sizeof(IdxT);      /* indices per 16-byte load */
     const int64_t nvec = ((uintptr_t)idx & 15) == 0 ? p0 / PER : 0;
@@ -370,14 +391,15 @@ int32_t zbalhip_layout_internal(const void *idx, int32_t idx_is_i64, int64_t tok
 
 /* ranks + offsets in one launch (no per-rank counts, no scratch) */
 int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
-                                      int32_t token_nums_type, int32_t *send_token_idx, int32_t *incl_i32,
-                                      int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed, hipStream_t st)
+                                      int32_t token_nums_type, const uint8_t *active_mask, int32_t *send_token_idx,
+                                      int32_t *incl_i32, int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed,
+                                      hipStream_t st)
 {
     const LayoutPlan p = plan_layout(tokens, topk, 64);
     layout_fused_kernel<int32_t><<<p.nblk, ZB_FUSED_THREADS, 0, st>>>(idx, (int)tokens, (int)topk, (int)experts,
                                                                     p.tokens_per_block, ceil_log2(experts), token_nums_type,
-                                                                    send_token_idx, incl_i32, row_off, counts_i64,
-                                                                    nums_typed);
+                                                                    active_mask, send_token_idx, incl_i32, row_off,
+                                                                    counts_i64, nums_typed);
     return zbalhip_check_launch();
 }
 

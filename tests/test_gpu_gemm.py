@@ -388,6 +388,35 @@ def test_fused_moe_shared_expert(buf, mode, share_i, smooth):
         assert np.array_equal(host(share), ref_share)
 
 
+@pytest.mark.parametrize("mode", [0, 2])
+@pytest.mark.parametrize("active", [0, 1, 37, 70])
+def test_fused_moe_active_mask(buf, mode, active):
+    """x_active_mask: the reference routes the first sum(mask) tokens and leaves everything else alone
+    (TokenActiveMaskCal, ...swiglu_quant_multistage_workspace.h:836-863; combine LocalWindowCopy,
+    zbal_moe_distribute_combine.h:724-760). The oracle is the unmasked layer on that prefix; the remaining output rows
+    must keep what they held."""
+    T, H, K, E, I = 70, 256, 4, 8, 128
+    x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 120 + mode)
+    mask = np.zeros(T, dtype=bool)
+    mask[rng(5).permutation(T)[:active]] = True          # only the count matters, not the positions
+    sentinel = torch.full((T, H), 7.0, dtype=torch.bfloat16, device="cuda")
+    sdt2 = torch.bfloat16 if mode == 0 else None
+    out, _, nums = buf.fused_deep_moe(dev(x, torch.bfloat16), dev(ids), buf.prepack_weight(dev(w1)), dev(s1),
+                                      buf.prepack_weight(dev(w2)), dev(s2, sdt2), dev(es), E, quant_mode=mode,
+                                      x_active_mask=dev(mask), out=sentinel)
+    got = host(out)
+    assert np.array_equal(got[active:], host(torch.full((T - active, H), 7.0, dtype=torch.bfloat16)))
+    if active == 0:
+        assert not host(nums).any()
+        return
+    ref, counts = zo.fused_moe(x[:active], zo.DT_BF16, ids[:active], es[:active], w1, s1, w2, s2, E, mode)
+    assert np.array_equal(host(nums), counts)
+    if mode == 2:
+        assert max_rel_err(zo.bf16_to_f32(got[:active]), zo.bf16_to_f32(ref)) < 2e-2
+    else:
+        assert np.array_equal(got[:active], ref)
+
+
 def test_fused_moe_empty_experts_and_invalid_ids(buf):
     T, H, K, E, I = 16, 256, 2, 32, 128                  # 32 picks over 32 experts: most experts are empty
     x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, 0, 90, zipf=1.2)
