@@ -120,7 +120,7 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             for (int s = 0; s < SLOTS; ++s) {
                 const int seg = s * blockDim.x + threadIdx.x;
                 if (seg < nseg) {
-                    __builtin_nontemporal_store(q[s], reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16));
+                    *reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16) = q[s];
                     if ((seg & 7) == 0) dest_scale[row * nblk128 + (seg >> 3)] = sc[s];
                 }
             }
@@ -150,7 +150,7 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             for (int s = 0; s < SLOTS; ++s) {
                 const int seg = s * blockDim.x + threadIdx.x;
                 if (seg < nseg)
-                    __builtin_nontemporal_store(q[s], reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16));
+                    *reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16) = q[s];
             }
             if (threadIdx.x == 0) dest_scale[row] = stored;
         }
@@ -181,7 +181,7 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
                 const int seg = s * blockDim.x + threadIdx.x;
                 if (seg < nseg) {
                     const u32x4 q = pack16_i8(sv[s], sq);
-                    __builtin_nontemporal_store(q, reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16));
+                    *reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16) = q;
                 }
             }
             if (threadIdx.x == 0) dest_scale[row] = stored;
@@ -213,7 +213,7 @@ permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ 
             for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u * blockDim.x + threadIdx.x;
                 if (c < nchunk)
-                    __builtin_nontemporal_store(v[u], reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)c * 8));
+                    *reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)c * 8) = v[u];
             }
         }
     }
