@@ -172,8 +172,11 @@ typedef struct {
  *   one byte per element: [E][N/128][K/128] blocks of 16 KiB; a block holds
  *     128 channels x 128 K-bytes, channel r at +128*r, and within a channel
  *     the 16-byte chunk c of its K-bytes at slot c ^ (r & 7) ^ ((r >> 3) & 1);
- *   INT4X2: [E, N, K/2] bytes; in each group of 8 consecutive k, byte b
- *     holds k[b] in the low and k[b+4] in the high nibble.
+ *   INT4X2: the same block order with 8 KiB blocks (128 channels x 128 k,
+ *     two values per byte); channel r at +64*r, and within a channel the
+ *     16-byte chunk c (k in [32c, 32c+32)) at slot c ^ ((r >> 2) & 3); in a
+ *     chunk, byte b of dword j holds k[8j+b] in the low and k[8j+4+b] in the
+ *     high nibble.
  */
 #define ZBAL_WEIGHT_FORMAT_ND      0 /* logical [E, K, N], N contiguous */
 #define ZBAL_WEIGHT_FORMAT_PREPACKED 1 /* made by zbal_moe_weight_prepack */

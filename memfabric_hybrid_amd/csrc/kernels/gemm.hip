@@ -35,19 +35,16 @@
 
 namespace {
 
-constexpr int BM = 128;          /* token rows per workgroup tile */
 constexpr int BN = 256;          /* output channels per workgroup tile */
-constexpr int BKB = 128;         /* K bytes per slab (128 int8/e4m3 elements) */
-constexpr int LDS_STRIDE = BKB + 16;
+constexpr int BKB = 128;         /* K bytes of an activation row per slab (128 int8/e4m3 elements) */
 constexpr int GROUP_N = 8;       /* channel tiles per schedule group */
-constexpr int kThreads = 256;
 
 enum { MODE_W8A8 = 1, MODE_FP8 = 2, MODE_W4A8 = 3 };
 
 struct GemmParams {
     const uint8_t *a;        /* [rows, K] */
     const float *a_scale;    /* [rows] or [rows, K/128] */
-    const uint8_t *w;        /* [E, N, K] or [E, N, K/2] */
+    const uint8_t *w;        /* pre-packed blocks, [E][N/128][K/128] x 16 KiB (8-bit) or 8 KiB (int4) */
     const void *wscale;
     const int32_t *row_off;  /* [E+1] */
     int experts;
@@ -64,62 +61,6 @@ struct GemmParams {
 struct TileCoord {
     int expert, m_tile, n_tile;
 };
-
-/* wave-uniform search of the logical tile this workgroup owns; false = nothing to do */
-template <int TILE_M>
-__device__ __forceinline__ bool locate_tile(const int32_t *__restrict__ row_off, int experts, int n_tiles,
-                                            TileCoord &tc)
-{
-    const int lane = threadIdx.x & 63;
-    int total = 0;
-    for (int base = 0; base < experts; base += 64) {
-        const int e = base + lane;
-        int t = 0;
-        if (e < experts) t = ((row_off[e + 1] - row_off[e] + TILE_M - 1) / TILE_M) * n_tiles;
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) t += __shfl_xor(t, off, 64);
-        total += t;
-    }
-    const int chunk = (total + 7) / 8;
-    const int slot = blockIdx.x >> 3, xcd = blockIdx.x & 7;
-    if (slot >= chunk) return false;
-    const int lid = xcd * chunk + slot;
-    if (lid >= total) return false;
-
-    int run = 0, expert = -1, start = 0, mt_e = 0;
-    for (int base = 0; base < experts; base += 64) {
-        const int e = base + lane;
-        int mt = 0;
-        if (e < experts) mt = (row_off[e + 1] - row_off[e] + TILE_M - 1) / TILE_M;
-        const int t = mt * n_tiles;
-        int incl = t;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int o = __shfl_up(incl, off, 64);
-            if (lane >= off) incl += o;
-        }
-        const int excl = run + incl - t;
-        const bool hit = t > 0 && lid >= excl && lid < excl + t;
-        const uint64_t bal = __ballot(hit);
-        if (bal) {
-            const int src = __ffsll((long long)bal) - 1;
-            expert = base + src;
-            start = __shfl(excl, src, 64);
-            mt_e = __shfl(mt, src, 64);
-            break;
-        }
-        run += __shfl(incl, 63, 64);
-    }
-    if (expert < 0) return false;
-    const int l = lid - start;
-    const int per_group = mt_e * GROUP_N;
-    const int ng = l / per_group;
-    const int r = l - ng * per_group;
-    tc.expert = expert;
-    tc.m_tile = r % mt_e;
-    tc.n_tile = ng * GROUP_N + r / mt_e;
-    return true;
-}
 
 __device__ __forceinline__ f32x4 mfma_fp8_16x16x128(const i32x8 &wfrag, const i32x8 &afrag)
 {
@@ -267,221 +208,9 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
     }
 }
 
-template <int MODE, bool GMM1, int OUT_DT>
-__global__ void __launch_bounds__(kThreads, 2)
-grouped_gemm_kernel(GemmParams p)
-{
-    __shared__ __attribute__((aligned(16))) uint8_t lds_a[BM * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) uint8_t lds_w[BN * LDS_STRIDE];
-    __shared__ __attribute__((aligned(16))) float lds_sa[BM];          /* fp8: activation scales of the slab */
-    __shared__ __attribute__((aligned(16))) float lds_gs[BN];          /* W4A8: group scales of the slab / 16 */
-    __shared__ float lds_rowmax[2][BM];
-
-    const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
-    TileCoord tc;
-    if (!locate_tile<BM>(p.row_off, p.experts, n_tiles, tc)) return;
-
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int wm = wave >> 1, wn = wave & 1;
-    const int row_begin = p.row_off[tc.expert] + tc.m_tile * BM;
-    const int row_end = p.row_off[tc.expert + 1];
-    const int K = p.K;
-    const int KB = K / 128;
-    const int I = p.N / 2;
-
-    /* ---- global -> register staging ------------------------------------------------ */
-    constexpr int A_LOADS = BM * (BKB / 16) / kThreads;                         /* 4 */
-    constexpr int W_BYTES_ROW = (MODE == MODE_W4A8) ? BKB / 2 : BKB;            /* bytes of one W row per slab */
-    constexpr int W_LOADS = BN * (W_BYTES_ROW / 16) / kThreads;                 /* 8 or 4 */
-    const uint8_t *a_ptr[A_LOADS];
-    const uint8_t *w_ptr[W_LOADS];
-    int a_lds[A_LOADS], w_lds[W_LOADS];
-#pragma unroll
-    for (int i = 0; i < A_LOADS; ++i) {
-        const int q = tid + i * kThreads, r = q >> 3, c = q & 7;
-        int gr = row_begin + r;
-        if (gr > p.max_rows - 1) gr = p.max_rows - 1;
-        a_ptr[i] = p.a + (int64_t)gr * K + c * 16;
-        a_lds[i] = r * LDS_STRIDE + c * 16;
-    }
-    const int64_t w_row_bytes = (MODE == MODE_W4A8) ? K / 2 : K;
-#pragma unroll
-    for (int i = 0; i < W_LOADS; ++i) {
-        constexpr int CPR = W_BYTES_ROW / 16; /* chunks per row */
-        const int q = tid + i * kThreads, r = q / CPR, c = q % CPR;
-        int wrow;
-        if (GMM1) wrow = (r < 128) ? tc.n_tile * 128 + r : I + tc.n_tile * 128 + (r - 128);
-        else wrow = tc.n_tile * BN + r;
-        w_ptr[i] = p.w + ((int64_t)tc.expert * p.N + wrow) * w_row_bytes + c * 16;
-        w_lds[i] = r * LDS_STRIDE + c * ((MODE == MODE_W4A8) ? 32 : 16);
-    }
-    /* per-slab scale staging */
-    const float *sa_ptr = nullptr;
-    if (MODE == MODE_FP8 && tid < BM) {
-        int gr = row_begin + tid;
-        if (gr > p.max_rows - 1) gr = p.max_rows - 1;
-        sa_ptr = p.a_scale + (int64_t)gr * KB;
-    }
-    const uint16_t *gs_ptr = nullptr;
-    if (MODE == MODE_W4A8) {
-        int wrow;
-        if (GMM1) wrow = (tid < 128) ? tc.n_tile * 128 + tid : I + tc.n_tile * 128 + (tid - 128);
-        else wrow = tc.n_tile * BN + tid;
-        gs_ptr = (const uint16_t *)p.wscale + (int64_t)tc.expert * KB * p.N + wrow;
-    }
-    /* fp8 weight block scales: two per slab for this tile */
-    const float *sw_ptr0 = nullptr, *sw_ptr1 = nullptr;
-    if (MODE == MODE_FP8) {
-        const int NB = p.N / 128;
-        const float *base = (const float *)p.wscale + (int64_t)tc.expert * KB * NB;
-        if (GMM1) { sw_ptr0 = base + tc.n_tile; sw_ptr1 = base + I / 128 + tc.n_tile; }
-        else { sw_ptr0 = base + tc.n_tile * 2; sw_ptr1 = sw_ptr0 + 1; }
-    }
-
-    u32x4 a_reg[A_LOADS], w_reg[W_LOADS];
-    float sa_reg = 0.0f, gs_reg = 0.0f;
-    auto fetch = [&](int kb) {
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) a_reg[i] = *reinterpret_cast<const u32x4 *>(a_ptr[i] + (int64_t)kb * BKB);
-#pragma unroll
-        for (int i = 0; i < W_LOADS; ++i)
-            w_reg[i] = *reinterpret_cast<const u32x4 *>(w_ptr[i] + (int64_t)kb * W_BYTES_ROW);
-        if (MODE == MODE_FP8 && tid < BM) sa_reg = sa_ptr[kb];
-        if (MODE == MODE_W4A8) gs_reg = zb_fp16_to_f32(gs_ptr[(int64_t)kb * p.N]) * 0.0625f;
-    };
-    auto stash = [&]() {
-#pragma unroll
-        for (int i = 0; i < A_LOADS; ++i) *reinterpret_cast<u32x4 *>(lds_a + a_lds[i]) = a_reg[i];
-#pragma unroll
-        for (int i = 0; i < W_LOADS; ++i) {
-            if constexpr (MODE == MODE_W4A8) {
-                /* byte b of each dword holds k[b] (low nibble) and k[b+4] (high nibble); <<4 keeps the sign
-                   and multiplies by 16, undone in the group scale */
-                u32x4 lo, hi;
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    lo[j] = (w_reg[i][j] << 4) & 0xf0f0f0f0u;
-                    hi[j] = w_reg[i][j] & 0xf0f0f0f0u;
-                }
-                u32x4 o0 = {lo[0], hi[0], lo[1], hi[1]};
-                u32x4 o1 = {lo[2], hi[2], lo[3], hi[3]};
-                *reinterpret_cast<u32x4 *>(lds_w + w_lds[i]) = o0;
-                *reinterpret_cast<u32x4 *>(lds_w + w_lds[i] + 16) = o1;
-            } else {
-                *reinterpret_cast<u32x4 *>(lds_w + w_lds[i]) = w_reg[i];
-            }
-        }
-        if (MODE == MODE_FP8 && tid < BM) lds_sa[tid] = sa_reg;
-        if (MODE == MODE_W4A8) lds_gs[tid] = gs_reg;
-    };
-
-    /* ---- accumulators ------------------------------------------------------------------ */
-    f32x4 accf[4][8];
-    i32x4 acci[4][8];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-        for (int nt = 0; nt < 8; ++nt) {
-            accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
-            acci[mt][nt] = i32x4{0, 0, 0, 0};
-        }
-
-    /* fragment addresses: lane reads row (lane%16) of a 16-row sub-tile, K bytes [32*(lane/16), +32) */
-    const int frag_row = lane & 15, frag_k = (lane >> 4) * 32;
-    int a_frag_off[4], w_frag_off[8];
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) a_frag_off[mt] = (wm * 64 + mt * 16 + frag_row) * LDS_STRIDE + frag_k;
-#pragma unroll
-    for (int nt = 0; nt < 8; ++nt) {
-        int r;
-        if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
-        else r = wn * 128 + nt * 16;
-        w_frag_off[nt] = (r + frag_row) * LDS_STRIDE + frag_k;
-    }
-
-    fetch(0);
-    for (int kb = 0; kb < KB; ++kb) {
-        __syncthreads();
-        stash();
-        __syncthreads();
-        if (kb + 1 < KB) fetch(kb + 1);
-
-        if constexpr (MODE == MODE_FP8) {
-            const float sw0 = sw_ptr0[(int64_t)kb * (p.N / 128)], sw1 = sw_ptr1[(int64_t)kb * (p.N / 128)];
-            i32x8 af[4];
-            float s0[4], s1[4];
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
-                const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds_a + a_frag_off[mt]);
-                const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds_a + a_frag_off[mt] + 16);
-                af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                const float sa = lds_sa[wm * 64 + mt * 16 + frag_row];
-                s0[mt] = sa * sw0;
-                s1[mt] = sa * sw1;
-            }
-#pragma unroll
-            for (int nt = 0; nt < 8; ++nt) {
-                const u32x4 lo = *reinterpret_cast<const u32x4 *>(lds_w + w_frag_off[nt]);
-                const u32x4 hi = *reinterpret_cast<const u32x4 *>(lds_w + w_frag_off[nt] + 16);
-                const i32x8 wf = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                const bool second = GMM1 ? (nt >= 4) : (wn == 1);
-#pragma unroll
-                for (int mt = 0; mt < 4; ++mt) {
-                    const f32x4 part = mfma_fp8_16x16x128(wf, af[mt]);
-                    const float s = second ? s1[mt] : s0[mt];
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], s, accf[mt][nt][i]);
-                }
-            }
-        } else {
-            /* int8 operands: two 64-deep MFMA steps per slab; lane's K bytes are [32*(lane/16) + 16*h, +16) */
-            i32x4 af[4][2];
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(lds_a + a_frag_off[mt] + 16 * h);
-                    af[mt][h] = i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
-                }
-#pragma unroll
-            for (int nt = 0; nt < 8; ++nt) {
-                i32x4 wf[2];
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const u32x4 v = *reinterpret_cast<const u32x4 *>(lds_w + w_frag_off[nt] + 16 * h);
-                    wf[h] = i32x4{(int)v[0], (int)v[1], (int)v[2], (int)v[3]};
-                }
-                if constexpr (MODE == MODE_W8A8) {
-#pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) {
-                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0], af[mt][0], acci[mt][nt], 0, 0, 0);
-                        acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[1], af[mt][1], acci[mt][nt], 0, 0, 0);
-                    }
-                } else {
-                    int r;
-                    if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
-                    else r = wn * 128 + nt * 16;
-                    const f32x4 gs = *reinterpret_cast<const f32x4 *>(&lds_gs[r + (lane >> 4) * 4]);
-#pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) {
-                        i32x4 part = i32x4{0, 0, 0, 0};
-                        part = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[0], af[mt][0], part, 0, 0, 0);
-                        part = __builtin_amdgcn_mfma_i32_16x16x64_i8(wf[1], af[mt][1], part, 0, 0, 0);
-#pragma unroll
-                        for (int i = 0; i < 4; ++i)
-                            accf[mt][nt][i] = __builtin_fmaf((float)part[i], gs[i], accf[mt][nt][i]);
-                    }
-                }
-            }
-        }
-    }
-
-    epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, row_begin, row_end, wm, wn, lane, &lds_rowmax[0][0], BM);
-}
-
 /* ------------------------------------------------------------------------------------------------------
- * Large-tile kernel for the 8-bit modes (W8A8, fp8): TM token rows x 256 channels x 128 K-bytes per
- * workgroup, TM/64 x 2 waves (same 64 x 128 wave tile as above), one workgroup per CU.
+ * The grouped GEMM kernel (W8A8, fp8, W4A8): TM token rows x 256 channels x 128 K elements per workgroup,
+ * TM/64 x 2 waves with a 64 x 128 wave tile each, one workgroup per CU.
  *
  * K slabs go from HBM to LDS without passing through registers: every wave issues
  * global_load_lds_dwordx4, which deposits the 64 lanes' 16-byte chunks in 1 KiB of consecutive LDS
@@ -497,23 +226,43 @@ grouped_gemm_kernel(GemmParams p)
  * 48 KiB is for few-row experts, where the job is to stream every weight byte once at HBM speed: it keeps
  * two weight slabs (64 KiB) in flight per CU and skips the MFMAs of 16-row groups past the expert's end.
  * Either way there is one barrier per step.
+ *
+ * W4A8: the weight slab stays packed in LDS (64 bytes per channel; block layout and nibble order as written by
+ * the pre-pack) and is unpacked to int8 * 16 in registers, a shift and two masks per packed dword; the factor 16
+ * is divided out of the accumulators, exactly, before the epilogue. Each 128-deep slab is one scale group:
+ * its 256 fp16 group scales ride along by DMA and `acc = fma(float(partial), gs, acc)` promotes the int32 partial.
  * ------------------------------------------------------------------------------------------------------ */
 constexpr int D_MAX_KB = 256;                 /* K up to 32768 */
 constexpr int D_MAX_EXPERTS = 1024;
 
-template <int TM, int NSTAGE>
+/* WRB = bytes of one weight row per slab: 128 (8-bit) or 64 (packed int4) */
+template <int TM, int NSTAGE, int WRB>
 struct DmaShape {
     static constexpr int ROW_GROUPS = TM / 64;
     static constexpr int NW = ROW_GROUPS * 2;
     static constexpr int THREADS = NW * 64;
     static constexpr int A_BYTES = TM * BKB;
-    static constexpr int STAGE_BYTES = (TM + BN) * BKB;
-    static constexpr int A_PARTS = TM / 8 / NW;      /* 1 KiB blocks of the A tile per wave (4) */
-    static constexpr int W_PARTS = BN / 8 / NW;      /* 1 KiB blocks of the W tile per wave (4 or 8) */
-    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 4 * D_MAX_KB * 4 + 2 * (D_MAX_EXPERTS + 1) * 4;
-    static_assert(A_PARTS == 4 && W_PARTS % 4 == 0, "issue schedule assumes four A blocks per wave");
+    static constexpr int W_BYTES = BN * WRB;
+    static constexpr int STAGE_BYTES = A_BYTES + W_BYTES;
+    static constexpr int HALF_BLOCKS = 128 * WRB / 1024;   /* 1 KiB blocks per 128-channel half: 16 or 8 */
+    static constexpr int A_PARTS = A_BYTES / 1024 / NW;    /* 1 KiB blocks of the A tile per wave (4) */
+    static constexpr int W_PARTS = W_BYTES / 1024 / NW;    /* 1 KiB blocks of the W tile per wave (2, 4 or 8) */
+    static constexpr int PARTS = W_PARTS > A_PARTS ? W_PARTS : A_PARTS;
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 4 * D_MAX_KB * 4 +
+                                     2 * (D_MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0);
+    static_assert(A_PARTS == 4 && PARTS % 4 == 0, "the issue schedule hands out a slab in four quarters");
+    static_assert(NW <= HALF_BLOCKS && HALF_BLOCKS % NW == 0, "a wave's W blocks must not straddle a weight half");
     static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
 };
+
+/* the pointer as scalar registers; a no-op where the compiler already knows it is wave-uniform */
+template <typename T>
+__device__ __forceinline__ const T *uniform_ptr(const T *p)
+{
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (const T *)(((uint64_t)hi << 32) | lo);
+}
 
 /*
  * One LDS-DMA transfer with the address split the way the instruction wants it: a wave-uniform 64-bit base in
@@ -524,7 +273,7 @@ __device__ __forceinline__ void dma16_sv(const uint8_t *uniform_base, uint32_t l
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
-                 : "s"(lds_wave_addr), "v"(lane_off), "s"(uniform_base)
+                 : "s"(lds_wave_addr), "v"(lane_off), "s"(uniform_ptr(uniform_base))
                  : "memory", "m0");
 }
 
@@ -532,7 +281,7 @@ __device__ __forceinline__ void dma4_sv(const float *uniform_base, uint32_t lane
 {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                  :
-                 : "s"(lds_wave_addr), "v"(lane_off_bytes), "s"(uniform_base)
+                 : "s"(lds_wave_addr), "v"(lane_off_bytes), "s"(uniform_ptr(uniform_base))
                  : "memory", "m0");
 }
 
@@ -541,13 +290,6 @@ __device__ __forceinline__ uint32_t lds_addr(const void *p)
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p;
 }
 
-template <typename T>
-__device__ __forceinline__ const T *uniform_ptr(const T *p)
-{
-    const uint64_t v = (uint64_t)p;
-    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
-    return (const T *)(((uint64_t)hi << 32) | lo);
-}
 
 /* wait until at most N of this wave's vector-memory operations are outstanding (they complete in order) */
 template <int N>
@@ -564,16 +306,19 @@ struct DmaTile {
     const uint8_t *a_base;            /* first K-byte of the tile's first activation row */
     const float *sa_base;             /* its fp8 block scales */
     const uint8_t *w_half[2];         /* K slab 0 of the tile's two 128-channel weight block rows */
+    const uint16_t *gs_mine;          /* W4A8: fp16 group scales, slab 0, of the weight half this wave brings in (wave % 2) */
 };
 
 template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
 __global__ void __launch_bounds__(TM * 2, 2)      /* TM/64 x 2 waves */
 grouped_gemm_dma_kernel(GemmParams p)
 {
-    static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8, "int4 weights need the register-staged kernel");
+    static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8 || MODE == MODE_W4A8, "unknown mode");
     static_assert(NSTAGE == 2 || NSTAGE == 3, "two or three stages");
-    using S = DmaShape<TM, NSTAGE>;
-    constexpr int NW = S::NW, STAGE_BYTES = S::STAGE_BYTES, A_BYTES = S::A_BYTES, W_PARTS = S::W_PARTS;
+    constexpr int WRB = MODE == MODE_W4A8 ? 64 : 128;
+    using S = DmaShape<TM, NSTAGE, WRB>;
+    constexpr int NW = S::NW, STAGE_BYTES = S::STAGE_BYTES, A_BYTES = S::A_BYTES, W_PARTS = S::W_PARTS, PARTS = S::PARTS;
+    constexpr int HALF_BLOCKS = S::HALF_BLOCKS, W_BLOCK_BYTES = 128 * WRB;     /* one 128-channel block of one slab */
     constexpr bool SKIP_ROW_GROUPS = TM < 256;      /* few-row shape: leave out the MFMAs of absent 16-row groups */
     using Tile = DmaTile;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
@@ -582,10 +327,11 @@ grouped_gemm_dma_kernel(GemmParams p)
     float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2 tiles][2][D_MAX_KB] fp8 weight block scales */
     int *lds_mtp = reinterpret_cast<int *>(lds_sw + 4 * D_MAX_KB);            /* [experts + 1] tiles of TM rows before expert e */
     int *lds_roff = lds_mtp + (D_MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
+    uint16_t *lds_gs = reinterpret_cast<uint16_t *>(lds_roff + (D_MAX_EXPERTS + 1));   /* [NSTAGE][BN] W4A8 group scales (fp16) */
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int wave_u = __builtin_amdgcn_readfirstlane(wave);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int wm = wave_u >> 1, wn = wave_u & 1;      /* wave-uniform, so everything derived from them lives in scalar registers */
     const int n_tiles = GMM1 ? (p.N / 2) / 128 : p.N / BN;
     const int K = p.K;
     const int KB = K / 128;
@@ -630,7 +376,7 @@ grouped_gemm_dma_kernel(GemmParams p)
     const int lid_end = (xcd + 1) * chunk < total ? (xcd + 1) * chunk : total;
     int lid = xcd * chunk + (blockIdx.x >> 3);
 
-    auto load_tile = [&](int id, Tile &t) {
+    auto load_tile = [&](int id, Tile &t) __attribute__((always_inline)) {
         t.valid = id < lid_end;
         if (!t.valid) return;
         const int q = id / n_tiles;                  /* index among all TM-row tiles: expert e has [mtp[e], mtp[e+1]) */
@@ -666,15 +412,19 @@ grouped_gemm_dma_kernel(GemmParams p)
         t.sa_base = p.a_scale + (int64_t)t.row_begin * KB;
         /* weights come pre-packed as 16 KiB blocks of 128 channels x 128 K-bytes in LDS order ([E][N/128][K/128]) */
         const int col0 = GMM1 ? t.n_tile : t.n_tile * 2, col1 = GMM1 ? I / 128 + t.n_tile : t.n_tile * 2 + 1;
-        t.w_half[0] = p.w + (((int64_t)expert * (p.N / 128) + col0) * KB) * 16384;
-        t.w_half[1] = p.w + (((int64_t)expert * (p.N / 128) + col1) * KB) * 16384;
+        t.w_half[0] = p.w + (((int64_t)expert * (p.N / 128) + col0) * KB) * W_BLOCK_BYTES;
+        t.w_half[1] = p.w + (((int64_t)expert * (p.N / 128) + col1) * KB) * W_BLOCK_BYTES;
+        if (MODE == MODE_W4A8) {      /* fp16 group scales [E][K/128][N]: the slab's 128 scales of each half are 256 bytes */
+            const uint16_t *gs = (const uint16_t *)p.wscale + (int64_t)expert * KB * p.N;
+            t.gs_mine = gs + ((wave_u & 1) ? col1 : col0) * 128;
+        }
     };
 
     /*
      * DMA: this wave fills 1 KiB blocks wave + NW*j of the A tile (j < 4) and of the W tile (j < W_PARTS). An A block is
      * tile rows 8*NW*j + r0 with r0 = 8*wave + lane/8, one swizzled 16-byte chunk per lane; rows past the expert's end
-     * are clamped onto its last row. 1 KiB block number b = wave + NW*j of the W tile is block b % 16 of
-     * the weight half b / 16, a straight copy. Addresses are a wave-uniform base plus a 32-bit lane offset.
+     * are clamped onto its last row. 1 KiB block number b = wave + NW*j of the W tile is block b % HALF_BLOCKS of
+     * the weight half b / HALF_BLOCKS, a straight copy. Addresses are a wave-uniform base plus a 32-bit lane offset.
      */
     const int r0 = 8 * wave + (lane >> 3);
     const uint32_t a_chunk = ((lane & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1))) * 16;
@@ -682,10 +432,14 @@ grouped_gemm_dma_kernel(GemmParams p)
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr(smem) + wave * 1024);     /* this wave's block 0 of stage 0 */
     const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave % S::ROW_GROUPS) * 256);
     const bool sa_wave = MODE == MODE_FP8 && wave < S::ROW_GROUPS;
-    /* part j of a slab: the wave's j-th block of the W tile, of the A tile (j < 4) and, with part 0, the activation scales */
-    auto issue_part = [&](const Tile &t, int kb, int stage, int j) {
+    const bool gs_wave = MODE == MODE_W4A8 && wave < 2;            /* wave h brings the group scales of weight half h */
+    const uint32_t lds_gs0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_gs) + (wave & 1) * 256);
+    /* part j of a slab: the wave's j-th block of the W tile (j < W_PARTS), of the A tile (j < 4) and, with part 0, the scales */
+    auto issue_part = [&](const Tile &t, int kb, int stage, int j) __attribute__((always_inline)) {
         const uint32_t dst = lds0 + stage * STAGE_BYTES + j * (NW * 1024);
-        dma16_sv(t.w_half[(NW * j) >> 4] + ((int64_t)kb * 16384 + ((NW * j) & 15) * 1024), w_off, dst + A_BYTES);
+        if (j < W_PARTS)
+            dma16_sv(t.w_half[(NW * j) / HALF_BLOCKS] + ((int64_t)kb * W_BLOCK_BYTES + ((NW * j) % HALF_BLOCKS) * 1024), w_off,
+                     dst + A_BYTES);
         if (j < 4) {
             /*
              * An 8-row block past the expert's end moves 16 bytes instead of 1 KiB (one lane): the transfer still
@@ -702,13 +456,15 @@ grouped_gemm_dma_kernel(GemmParams p)
             if (rel > t.last_rel) rel = t.last_rel;
             dma4_sv(t.sa_base + kb, (uint32_t)rel * (uint32_t)KB * 4u, lds_sa0 + stage * TM * 4);
         }
+        if (j == 0 && gs_wave)      /* 128 fp16 scales = 64 dwords, one per lane */
+            dma4_sv((const float *)(t.gs_mine + (int64_t)kb * p.N), lane * 4u, lds_gs0 + stage * (BN * 2));
     };
-    auto issue = [&](const Tile &t, int kb, int stage) {
+    auto issue = [&](const Tile &t, int kb, int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < W_PARTS; ++j) issue_part(t, kb, stage, j);
+        for (int j = 0; j < PARTS; ++j) issue_part(t, kb, stage, j);
     };
     /* the two weight block scales of every K slab of a tile go to LDS by DMA as well: lane = K slab */
-    auto issue_sw = [&](const Tile &t, int buf) {
+    auto issue_sw = [&](const Tile &t, int buf) __attribute__((always_inline)) {
         if (MODE != MODE_FP8) return;
         const int sw_stride = p.N / 128;
         const float *base = (const float *)p.wscale + (int64_t)t.expert * KB * sw_stride;
@@ -724,19 +480,24 @@ grouped_gemm_dma_kernel(GemmParams p)
     };
     /* this wave's vector-memory operations per slab: what may stay outstanding while an older slab is awaited */
     constexpr int OPS = W_PARTS + 4;
+    const bool extra_op_wave = sa_wave || gs_wave;                  /* one more operation per slab: the scales */
 
     /* fragment reads: row lane%16 of a 16-row sub-tile, logical chunks 2*(lane/16) and 2*(lane/16)+1 */
     const int frag_row = lane & 15;
     const int key = (lane & 7) ^ ((lane >> 3) & 1), g2 = (lane >> 4) * 2;
     const int off_lo = frag_row * BKB + ((g2 ^ key) * 16), off_hi = frag_row * BKB + (((g2 + 1) ^ key) * 16);
-    int w_sub[8];
+    /* int4: one 16-byte chunk per lane, chunk lane/16 of channel lane%16 of the 16-channel block, at its swizzled slot */
+    const int w4_off = frag_row * 64 + (((lane >> 4) ^ ((frag_row >> 2) & 3)) * 16);
+    int w_sub[8], w_ch[8];
 #pragma unroll
     for (int nt = 0; nt < 8; ++nt) {
         int r;
         if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
         else r = wn * 128 + nt * 16;
-        w_sub[nt] = A_BYTES + r * BKB;
+        w_sub[nt] = A_BYTES + r * WRB;
+        w_ch[nt] = r;                             /* tile-local index of the sub-tile's first output channel */
     }
+    const int lane_ch = (lane >> 4) * 4;          /* the lane's four channels within a sub-tile */
 
     Tile cur, nxt;
     load_tile(lid, cur);
@@ -770,7 +531,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             /* the slab after this one exists if the tile or the sequence goes on; its loads may stay in flight */
             const bool later = kb + 1 < KB || nxt.valid;
             if (NSTAGE == 3 && later) {
-                if (sa_wave) wait_vmcnt<OPS + 1>();
+                if (extra_op_wave) wait_vmcnt<OPS + 1>();
                 else wait_vmcnt<OPS>();
             } else {
                 wait_vmcnt<0>();
@@ -793,9 +554,9 @@ grouped_gemm_dma_kernel(GemmParams p)
                 if (more) issue(ft, fill_kb, fill_stage);
                 continue;
             }
-            auto issue_quarter = [&](int q) {
+            auto issue_quarter = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
-                for (int j = q * (W_PARTS / 4); j < (q + 1) * (W_PARTS / 4); ++j) issue_part(ft, fill_kb, fill_stage, j);
+                for (int j = q * (PARTS / 4); j < (q + 1) * (PARTS / 4); ++j) issue_part(ft, fill_kb, fill_stage, j);
             };
 
             auto load_w = [&](int nt) -> i32x8 {
@@ -845,6 +606,51 @@ grouped_gemm_dma_kernel(GemmParams p)
                     }
                     wf = wf_n;
                 }
+            } else if constexpr (MODE == MODE_W4A8) {
+                /*
+                 * The lane's 16 packed bytes are its 32 K values of this slab: dwords 0-1 unpack into the operand of the
+                 * first 64-deep MFMA, dwords 2-3 into the second (times 16: the nibble moves to the top of its byte,
+                 * which keeps the sign). The pair's int32 sum is promoted with the slab's group scales, and as in the
+                 * fp8 mode the MFMAs of pair p+1 are issued before the conversions and FMAs of pair p.
+                 */
+                const uint16_t *gsb = lds_gs + cur_stage * BN;
+                auto load_pk = [&](int nt) -> u32x4 { return *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + w4_off); };
+                auto load_gs = [&](int nt) -> u32x2 { return *reinterpret_cast<const u32x2 *>(gsb + lane_ch + w_ch[nt]); };
+                auto lo4 = [](uint32_t v) -> int { return (int)((v << 4) & 0xf0f0f0f0u); };
+                auto hi4 = [](uint32_t v) -> int { return (int)(v & 0xf0f0f0f0u); };
+                auto mfma_pair = [&](const u32x4 &pk, const i32x8 &a) -> i32x4 {
+                    const i32x4 w0 = i32x4{lo4(pk[0]), hi4(pk[0]), lo4(pk[1]), hi4(pk[1])};
+                    const i32x4 w1 = i32x4{lo4(pk[2]), hi4(pk[2]), lo4(pk[3]), hi4(pk[3])};
+                    i32x4 part = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, i32x4{a[0], a[1], a[2], a[3]}, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                    return __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, i32x4{a[4], a[5], a[6], a[7]}, part, 0, 0, 0);
+                };
+                /* the packed chunk and the raw fp16 scales of the next channel sub-tile are fetched one sub-tile ahead */
+                u32x4 pk = load_pk(0);
+                u32x2 gsr = load_gs(0);
+                i32x4 part = mfma_pair(pk, af[0]);
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt) {
+                    u32x4 pkn = pk;
+                    u32x2 gsn = gsr;
+                    if (nt + 1 < 8) {
+                        pkn = load_pk(nt + 1);
+                        gsn = load_gs(nt + 1);
+                    }
+                    if (nt < 4 && more) issue_quarter(nt);
+                    const float gs[4] = {zb_fp16_to_f32(gsr[0] & 0xffffu), zb_fp16_to_f32(gsr[0] >> 16),
+                                         zb_fp16_to_f32(gsr[1] & 0xffffu), zb_fp16_to_f32(gsr[1] >> 16)};
+#pragma unroll
+                    for (int mt = 0; mt < 4; ++mt) {
+                        i32x4 nxt_part = part;
+                        if (mt < 3) nxt_part = mfma_pair(pk, af[mt + 1]);
+                        else if (nt + 1 < 8) nxt_part = mfma_pair(pkn, af[0]);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf((float)part[i], gs[i], accf[mt][nt][i]);
+                        part = nxt_part;
+                    }
+                    pk = pkn;
+                    gsr = gsn;
+                }
             } else {
                 /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
 #pragma unroll
@@ -864,6 +670,14 @@ grouped_gemm_dma_kernel(GemmParams p)
                                 wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
                 }
             }
+        }
+        if constexpr (MODE == MODE_W4A8) {      /* the unpacked weights were 16 x their value; a power of two divides out exactly */
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                for (int nt = 0; nt < 8; ++nt)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) accf[mt][nt][i] *= 0.0625f;
         }
         TileCoord tc;
         tc.expert = cur.expert;
@@ -915,7 +729,7 @@ inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles, int til
 template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
 int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
 {
-    using S = DmaShape<TM, NSTAGE>;
+    using S = DmaShape<TM, NSTAGE, MODE == MODE_W4A8 ? 64 : 128>;
     static int cus[64] = {};
     const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE>);
     int dev = 0;
@@ -974,7 +788,8 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
         const int32_t rc = launch_dma<MODE_W8A8, true, ZDT_BF16>(p, n_tiles, st);
         if (rc != ZBALHIP_OK) return rc;
     } else {
-        grouped_gemm_kernel<MODE_W4A8, true, ZDT_BF16><<<grid_for(max_rows, experts, n_tiles, BM), kThreads, 0, st>>>(p);
+        const int32_t rc = launch_dma<MODE_W4A8, true, ZDT_BF16>(p, n_tiles, st);
+        if (rc != ZBALHIP_OK) return rc;
     }
     int64_t rb = max_rows < 4096 ? max_rows : 4096;
     requant_rows_kernel<<<(unsigned)rb, 256, 0, st>>>(sgl_ws, p.rowmax, row_off, (int)experts, (int)(n1 / 2),
@@ -1006,8 +821,5 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
         return bf ? launch_dma<MODE_W8A8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_W8A8, false, ZDT_FP16>(p, n_tiles, st);
     if (mode == MODE_FP8)
         return bf ? launch_dma<MODE_FP8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_FP8, false, ZDT_FP16>(p, n_tiles, st);
-    const unsigned grid = grid_for(max_rows, experts, n_tiles, BM);
-    if (bf) grouped_gemm_kernel<MODE_W4A8, false, ZDT_BF16><<<grid, kThreads, 0, st>>>(p);
-    else grouped_gemm_kernel<MODE_W4A8, false, ZDT_FP16><<<grid, kThreads, 0, st>>>(p);
-    return zbalhip_check_launch();
+    return bf ? launch_dma<MODE_W4A8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_W4A8, false, ZDT_FP16>(p, n_tiles, st);
 }

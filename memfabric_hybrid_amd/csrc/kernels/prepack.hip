@@ -10,15 +10,13 @@
  * is then two runs of consecutive addresses, and each LDS-DMA instruction
  * copies 1 KiB of consecutive bytes.
  *
- * int4 weights: [E, N, K/2], two values per byte (64x64 tiles transposed
- * through LDS).
+ * int4 weights: the same block order with 8 KiB blocks, two values per
+ * byte (details at the kernel).
  */
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
 
 namespace {
-
-constexpr int kTile = 64;
 
 __global__ void __launch_bounds__(256)
 tile_swizzle_bytes_kernel(const uint8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
@@ -46,30 +44,40 @@ tile_swizzle_bytes_kernel(const uint8_t *__restrict__ src, int64_t K, int64_t N,
 }
 
 /*
- * int8 values in [-8,7], [E,K,N] -> [E,N,K/2] bytes. Within every group of 8 consecutive k, byte b (0..3)
- * holds k[b] in its low nibble and k[b+4] in its high nibble, so that the GEMM unpacks a dword into two
- * dwords of four consecutive k each with one shift and two masks.
+ * int8 values in [-8,7], [E,K,N] -> [E][N/128][K/128] blocks of 8 KiB, two values per byte. A block holds 128
+ * channels x 128 k as the GEMM wants them in LDS: channel r at +64*r, and within it the 16-byte chunk c (k in
+ * [32c, 32c+32)) in slot c ^ ((r >> 2) & 3), so that the 64 lanes of a fragment read (16 channels x 4 chunks)
+ * touch 64 distinct slots. Within a chunk, byte b of dword j holds k[8j+b] in its low nibble and k[8j+4+b] in
+ * its high nibble: the GEMM unpacks a dword into two dwords of four consecutive k with one shift and two masks.
  */
 __global__ void __launch_bounds__(256)
-transpose_pack_int4_kernel(const int8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
+tile_pack_int4_kernel(const int8_t *__restrict__ src, int64_t K, int64_t N, uint8_t *__restrict__ dst)
 {
-    __shared__ int8_t tile[kTile][kTile + 4];
+    __shared__ int8_t tile[128][128 + 16];           /* [k][n] */
     const int64_t e = blockIdx.z;
-    const int64_t k0 = (int64_t)blockIdx.y * kTile, n0 = (int64_t)blockIdx.x * kTile;
+    const int64_t k0 = (int64_t)blockIdx.y * 128, n0 = (int64_t)blockIdx.x * 128;
     const int8_t *s = src + e * K * N;
-    uint8_t *d = dst + e * (K / 2) * N;
-    for (int i = threadIdx.x; i < kTile * kTile; i += blockDim.x) {
-        const int kk = i / kTile, nn = i % kTile;
-        tile[kk][nn] = (k0 + kk < K && n0 + nn < N) ? s[(k0 + kk) * N + n0 + nn] : (int8_t)0;
+    for (int i = threadIdx.x; i < 128 * 8; i += blockDim.x) {
+        const int kk = i >> 3, c = i & 7;
+        *reinterpret_cast<u32x4 *>(&tile[kk][c * 16]) = *reinterpret_cast<const u32x4 *>(s + (k0 + kk) * N + n0 + c * 16);
     }
     __syncthreads();
-    for (int i = threadIdx.x; i < kTile * kTile / 2; i += blockDim.x) {
-        const int nn = i / (kTile / 2), kp = i % (kTile / 2);
-        const int kl = (kp / 4) * 8 + (kp % 4); /* k of the low nibble; the high nibble is kl + 4 */
-        if (k0 + kl + 4 < K && n0 + nn < N) {
-            const uint32_t lo = (uint32_t)tile[kl][nn] & 0xfu, hi = (uint32_t)tile[kl + 4][nn] & 0xfu;
-            d[(n0 + nn) * (K / 2) + (k0 / 2) + kp] = (uint8_t)(lo | (hi << 4));
+    uint8_t *d = dst + ((e * (N / 128) + blockIdx.x) * (K / 128) + blockIdx.y) * 8192;
+    for (int i = threadIdx.x; i < 512; i += blockDim.x) {       /* one 16-byte chunk per iteration */
+        const int r = i >> 2, c = i & 3;
+        uint32_t w[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            w[j] = 0;
+#pragma unroll
+            for (int bb = 0; bb < 4; ++bb) {
+                const uint32_t lo = (uint32_t)tile[32 * c + 8 * j + bb][r] & 0xfu;
+                const uint32_t hi = (uint32_t)tile[32 * c + 8 * j + 4 + bb][r] & 0xfu;
+                w[j] |= (lo | (hi << 4)) << (8 * bb);
+            }
         }
+        const int slot = c ^ (((r & 15) >> 2) & 3);
+        *reinterpret_cast<u32x4 *>(d + (r >> 4) * 1024 + (r & 15) * 64 + slot * 16) = u32x4{w[0], w[1], w[2], w[3]};
     }
 }
 
@@ -80,15 +88,10 @@ extern "C" int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int6
 {
     if (!src || !dst || src == dst || experts <= 0 || k <= 0 || n <= 0) return ZBALHIP_INVALID;
     if (experts > 65535) return ZBALHIP_INVALID;
-    if (to_int4) {
-        if ((k % 8) != 0 || (k + kTile - 1) / kTile > 65535) return ZBALHIP_INVALID;
-        dim3 grid((unsigned)((n + kTile - 1) / kTile), (unsigned)((k + kTile - 1) / kTile), (unsigned)experts);
-        transpose_pack_int4_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const int8_t *)src, k, n, (uint8_t *)dst);
-    } else {
-        if ((k % 128) != 0 || (n % 128) != 0 || k / 128 > 65535) return ZBALHIP_INVALID;
-        if (((uintptr_t)src & 15) != 0 || ((uintptr_t)dst & 15) != 0) return ZBALHIP_INVALID;
-        dim3 grid((unsigned)(n / 128), (unsigned)(k / 128), (unsigned)experts);
-        tile_swizzle_bytes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t *)src, k, n, (uint8_t *)dst);
-    }
+    if ((k % 128) != 0 || (n % 128) != 0 || k / 128 > 65535) return ZBALHIP_INVALID;
+    if (((uintptr_t)src & 15) != 0 || ((uintptr_t)dst & 15) != 0) return ZBALHIP_INVALID;
+    dim3 grid((unsigned)(n / 128), (unsigned)(k / 128), (unsigned)experts);
+    if (to_int4) tile_pack_int4_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const int8_t *)src, k, n, (uint8_t *)dst);
+    else tile_swizzle_bytes_kernel<<<grid, 256, 0, (hipStream_t)stream>>>((const uint8_t *)src, k, n, (uint8_t *)dst);
     return zbalhip_check_launch();
 }

@@ -292,10 +292,15 @@ def test_weight_prepack(buf):
         want[:, :, :, r, slot, :] = wt[:, :, :, r, slot ^ f, :]
     assert np.array_equal(packed, want)
     assert buf.lib.zbalhip_weight_prepack(dev(w).data_ptr(), E, 200, 136, 0, dev(w).data_ptr() + 16, None) != 0
-    N = 136
-    K = 256
+    # int4: 8 KiB blocks of 128 channels x 128 k; channel r at +64*r, the 16-byte chunk c (k in [32c, 32c+32)) in slot
+    # c ^ ((r >> 2) & 3) (r taken within its 16-channel group); byte b of dword j = k[8j+b] | k[8j+4+b] << 4
     w4 = rng(41).integers(-8, 8, (E, K, N)).astype(np.int8)
-    p4 = host(buf.prepack_weight(dev(w4), int4=True))
-    wt = w4.transpose(0, 2, 1).reshape(E, N, K // 8, 8)
-    want = ((wt[..., :4] & 0xf) | ((wt[..., 4:] & 0xf) << 4)).astype(np.uint8).reshape(E, N, K // 2)
-    assert np.array_equal(p4, want)
+    p4 = host(buf.prepack_weight(dev(w4), int4=True)).reshape(E, N // 128, K // 128, 128, 4, 16)
+    wt = w4.transpose(0, 2, 1).reshape(E, N // 128, 128, K // 128, 4, 4, 2, 4)       # [e][nb][r][kb][c][j][half][b]
+    nib = ((wt[..., 0, :] & 0xf) | ((wt[..., 1, :] & 0xf) << 4)).astype(np.uint8)     # [e][nb][r][kb][c][j][b]
+    nib = nib.reshape(E, N // 128, 128, K // 128, 4, 16).transpose(0, 1, 3, 2, 4, 5)  # [e][nb][kb][r][c][16]
+    f4 = ((r & 15) >> 2) & 3
+    want4 = np.empty_like(nib)
+    for slot in range(4):
+        want4[:, :, :, r, slot, :] = nib[:, :, :, r, slot ^ f4, :]
+    assert np.array_equal(p4, want4)
