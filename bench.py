@@ -37,7 +37,7 @@ PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # HBM bytes one GMM1 launch moves at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from two
 # `rocprofv3 --pmc` runs of this script (summary and counter calibration: profiles/moe_prefill_fp8_kernels.txt)
-GMM1_TRAFFIC_BYTES_T4096 = 3.312e9
+GMM1_TRAFFIC_BYTES_T4096 = 3.677e9
 REDUCE_TRAFFIC_BYTES = 2.416e9  # 2.0 x 1048607 KiB + 262144 KiB (profiles/reduce_8x256MiB.txt)
 
 
@@ -225,7 +225,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": wbytes1 / t1 / 1e9 / PEAK_HBM_GBS, "traffic": None,
                     "experts_with_tokens": touched}
     else:
-        kname = "grouped_gemm_dma_kernel<fp8, gmm1>" if mode == 2 else "grouped_gemm_kernel<w4a8, gmm1>"
+        kname = "grouped_gemm_dma_kernel<fp8, gmm1>" if mode == 2 else "grouped_gemm_dma_kernel<w4a8, gmm1>"
         roofline = {"kernel": kname, "bound": "mfma", "achieved": flops1 / t1 / 1e12,
                     "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s" if mode == 2 else "TOP/s",
                     "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
