@@ -142,6 +142,15 @@ ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, 
                                     int32_t *scratch, int32_t scratch_blocks, void *stream);
 
 /*
+ * OR-ed into `mode` of the two grouped GEMMs: `w1`/`w2` and their scales are
+ * not one stacked tensor each but device arrays of `experts` 64-bit addresses,
+ * entry e = expert e's pre-packed weights / its scales (16-byte aligned;
+ * the reference's EXEC_FLAG_TENSOR_LIST,
+ * …swiglu_quant_multistage_workspace.h:669-673, 755-757, 1531-1558).
+ */
+#define ZBALHIP_WEIGHTS_AS_LISTS 0x100
+
+/*
  * Grouped GEMM 1 with dequant + SwiGLU + requant epilogue (AIC loop
  * …swiglu_quant_multistage_workspace.h:603-833, epilogue
  * block_epilogue_per_token_dequant_swiglu.h:171-298, BlockQuant

@@ -109,8 +109,12 @@ int32_t zbal_combine_low_latency(const zbal_tensor_info_t *expandX, const zbal_t
  * expert's, optional shareSmoothScales [H]; its result goes to shareOutput
  * [tokens, H] and is not added to output. Pass all of them or none.
  * xActiveMask [tokens] (one byte per token): only the first sum(mask)
- * tokens are routed and written, as in the reference. isTensorList != 0 is
- * rejected with -2.
+ * tokens are routed and written, as in the reference. isTensorList != 0
+ * (EXEC_FLAG_TENSOR_LIST in the reference kernel): `data` of gmm1Weight,
+ * gmm1Scale, gmm2Weight and gmm2Scale is a device array of moeExpertNum
+ * 64-bit addresses, entry e = expert e's own pre-packed weight / scale tensor
+ * (16-byte aligned); dataType, shape and format still describe the stacked
+ * tensor. The shared expert's operands are always plain tensors.
  */
 int32_t zbal_fused_deep_moe(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds,
                             const zbal_tensor_info_t *gmm1Weight, const zbal_tensor_info_t *gmm1Scale,

@@ -86,6 +86,7 @@ class Buffer:
         self.lib = capi.load()
         self.comm = _acquire(self.device.index or 0)
         self.send_token_idx = None       # kept between layout, dispatch and combine (zbal_deepep.cpp:254,305,423)
+        self._tables = {}                # device address tables of tensor-list operands
         self._closed = False
 
     def close(self):
@@ -106,6 +107,27 @@ class Buffer:
     @staticmethod
     def _ti(t, **kw):
         return ctypes.byref(capi.tensor_info(t, **kw))
+
+    def _list_ti(self, seq, num_experts, **kw):
+        """Descriptor of a tensor list: shape and type of the stacked tensor, `data` = a device table of the
+        per-expert addresses (kept in a small cache, so repeated calls with the same tensors copy nothing)."""
+        if len(seq) != num_experts:
+            raise ValueError("a tensor list needs one tensor per expert")
+        first = seq[0]
+        per = tuple(first.shape[1:]) if first.shape[0] == 1 and first.dim() == 3 else tuple(first.shape)
+        for t in seq:
+            if not t.is_contiguous() or t.dtype != first.dtype or t.numel() != first.numel():
+                raise ValueError("tensor-list entries must be contiguous and alike")
+        key = tuple(t.data_ptr() for t in seq)
+        table = self._tables.get(key)
+        if table is None:
+            if len(self._tables) >= 64:
+                self._tables.clear()
+            table = torch.tensor(key, dtype=torch.int64).to(self.device)
+            self._tables[key] = table
+        ti = capi.tensor_info(first, shape=(num_experts,) + per, **kw)
+        ti.data = table.data_ptr()
+        return ctypes.byref(ti)
 
     # -- router (extension) ------------------------------------------------------------------
     def topk_route(self, logits, num_topk):
@@ -244,14 +266,15 @@ class Buffer:
     def fused_deep_moe(self, x, topk_idx, gmm1_permuted_weight, gmm1_permuted_weight_scale, gmm2_weight,
                        gmm2_weight_scale, topk_weights, num_experts, quant_mode=0, expert_smooth_scales=None,
                        share_gmm1_weight=None, share_gmm1_scale=None, share_gmm2_weight=None, share_gmm2_scale=None,
-                       share_smooth_scales=None, x_active_mask=None, workspace=None, out=None):
+                       share_smooth_scales=None, x_active_mask=None, workspace=None, out=None, is_tensor_list=False):
         """zbal_deepep.cpp:658-802. Weights are pre-packed (prepack_weight; shared-expert weights as [1,N,K]).
         Returns (output, share_output, expert_token_nums) like the reference; share_output is None without a shared
         expert. x_active_mask [T] bool: only the first sum(mask) tokens are routed; the other rows of `out` keep
-        their contents."""
+        their contents. is_tensor_list: the four routed-expert operands are sequences of per-expert tensors (each
+        pre-packed on its own, [1,N,K] or [N,K]); the library receives one device table of addresses per operand."""
         T, H = x.shape
         K = topk_idx.shape[1]
-        n1 = gmm1_permuted_weight.shape[1]
+        n1 = gmm1_permuted_weight[0].shape[-2] if is_tensor_list else gmm1_permuted_weight.shape[1]
         shared = share_gmm1_weight is not None
         sn1 = share_gmm1_weight.shape[-2] if shared else 0
         expert_ids = topk_idx if topk_idx.dtype == torch.int32 else topk_idx.to(torch.int32)
@@ -263,11 +286,16 @@ class Buffer:
         token_nums = self._empty((num_experts,), torch.int64)
         wdt = {0: None, 1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[quant_mode]
         null = ctypes.byref(capi.TensorInfo())
+        if is_tensor_list:
+            def wti(t, **kw):
+                return self._list_ti(t, num_experts, **kw)
+        else:
+            wti = self._ti
         capi.check("zbal_fused_deep_moe", self.lib.zbal_fused_deep_moe(
             self._ti(x), self._ti(expert_ids),
-            self._ti(gmm1_permuted_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED),
-            self._ti(gmm1_permuted_weight_scale),
-            self._ti(gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), self._ti(gmm2_weight_scale),
+            wti(gmm1_permuted_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED),
+            wti(gmm1_permuted_weight_scale),
+            wti(gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), wti(gmm2_weight_scale),
             self._ti(topk_weights), self._ti(expert_smooth_scales) if expert_smooth_scales is not None else null,
             self._ti(share_gmm1_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED) if shared else null,
             self._ti(share_gmm1_scale) if shared else null,
@@ -276,5 +304,5 @@ class Buffer:
             self._ti(share_smooth_scales) if share_smooth_scales is not None else null,
             self._ti(x_active_mask.view(torch.uint8)) if x_active_mask is not None else null,
             self._ti(out), self._ti(share_out) if shared else null, self._ti(token_nums), self._ti(workspace),
-            num_experts, quant_mode, 0, n1, sn1, 0, self.comm, capi.stream_ptr(), 0))
+            num_experts, quant_mode, 0, n1, sn1, int(is_tensor_list), self.comm, capi.stream_ptr(), 0))
         return out, share_out, token_nums

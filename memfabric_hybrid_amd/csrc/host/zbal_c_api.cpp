@@ -2,10 +2,9 @@
  * Outer C ABI of the operator layer: argument validation, handle lookup and
  * the virtual call into the communicator's backend. Validation order and
  * return codes follow the reference's zbal_operations.cpp (lines cited per
- * function); two deliberate differences: the communicator handle is looked
+ * function); one deliberate difference: the communicator handle is looked
  * up in the registry before use (the reference casts it blindly and its MoE
- * entry points do not even check it for null, :283-286, :308-311), and the
- * shared-expert / tensor-list operands of the fused operator are rejected.
+ * entry points do not even check it for null, :283-286, :308-311).
  */
 #include <cstring>
 #include <initializer_list>
@@ -278,13 +277,12 @@ ZBAL_API int32_t zbal_fused_deep_moe(
     auto present = [](const zbal_tensor_info_t *t) { return t != nullptr && t->data != nullptr; };
     const bool shared = present(shareGmm1Weight);
     ZBAL_VALIDATE_RETURN(shared == present(shareGmm1Scale) && shared == present(shareGmm2Weight) && shared == present(shareGmm2Scale) && shared == present(shareOutput) && shared == (shareGmm1HLen > 0) && (shared || !present(shareSmoothScales)), "FusedDeepMoe failed as the shared expert needs both weights, both scales, shareOutput and shareGmm1HLen > 0, or none of them", Z_INVALID_PARAM);
-    ZBAL_VALIDATE_RETURN(isTensorList == 0, "FusedDeepMoe failed as tensor-list weights are not supported", Z_INVALID_PARAM);
     CommunicatorPtr c = Resolve("FusedDeepMoe", comm);
     if (!c) return Z_INVALID_PARAM;
     return c->FusedDeepMoe(x, expertIds, gmm1Weight, gmm1Scale, gmm2Weight, gmm2Scale, expertScales, expertSmoothScales,
                            shareGmm1Weight, shareGmm1Scale, shareGmm2Weight, shareGmm2Scale, shareSmoothScales, xActiveMask,
                            output, shareOutput, expertTokenNums, workspace, moeExpertNum, quantMode, globalBs, gmm1HLen,
-                           shareGmm1HLen, stream, flags);
+                           shareGmm1HLen, isTensorList != 0, stream, flags);
 }
 
 /* ---- extensions -------------------------------------------------------------------------- */

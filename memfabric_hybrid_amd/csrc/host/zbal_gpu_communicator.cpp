@@ -415,7 +415,7 @@ public:
                          const zbal_tensor_info_t *output, const zbal_tensor_info_t *shareOutput,
                          const zbal_tensor_info_t *expertTokenNums, const zbal_tensor_info_t *workspace,
                          int64_t moeExpertNum, int64_t quantMode, int64_t, int64_t gmm1HLen, int64_t shareGmm1HLen,
-                         aclrtStream stream, int64_t) override
+                         bool isTensorList, aclrtStream stream, int64_t) override
     {
         const char *op = "FusedDeepMoe";
         if (!SingleRank(op)) return Z_INVALID_PARAM;
@@ -484,6 +484,8 @@ public:
         float *sgl = mode == 2 ? nullptr : (float *)(base + ws.sgl);
         void *y = base + ws.y;
         const int qmode = mode == 2 ? 2 : 1;
+        /* tensor lists: the four routed-expert descriptors point at device tables of one address per expert */
+        const int32_t gemmMode = mode | (isTensorList ? ZBALHIP_WEIGHTS_AS_LISTS : 0);
         if (T == 0) { /* nothing routed: counts are zero */
             return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth,
                                                             nullptr, 0, H, K, E, qmode, q1, xs, expandIdx,
@@ -516,10 +518,10 @@ public:
                                          qmode, q1, xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff, scratch,
                                          ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
         if (rc != 0) return Launched(op, rc);
-        rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1, mode, q2, scale2,
-                                       sgl, stream);
+        rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1, gemmMode, q2,
+                                       scale2, sgl, stream);
         if (rc != 0) return Launched(op, rc);
-        rc = zbalhip_gmm2_dequant(q2, scale2, gmm2Weight->data, gmm2Scale->data, wscale2Dt, rowOff, E, rows, I, H, mode,
+        rc = zbalhip_gmm2_dequant(q2, scale2, gmm2Weight->data, gmm2Scale->data, wscale2Dt, rowOff, E, rows, I, H, gemmMode,
                                   x->dataType, y, stream);
         if (rc != 0) return Launched(op, rc);
         return Launched(op, zbalhip_combine(y, x->dataType, rowOff, 0, (const float *)expertScales->data,

@@ -169,7 +169,7 @@ public:
                                  const zbal_tensor_info_t *output, const zbal_tensor_info_t *shareOutput,
                                  const zbal_tensor_info_t *expertTokenNums, const zbal_tensor_info_t *workspace,
                                  int64_t moeExpertNum, int64_t quantMode, int64_t globalBs, int64_t gmm1HLen,
-                                 int64_t shareGmm1HLen, aclrtStream stream, int64_t flags) = 0;
+                                 int64_t shareGmm1HLen, bool isTensorList, aclrtStream stream, int64_t flags) = 0;
     virtual int32_t TopkRoute(const zbal_tensor_info_t *logits, int64_t topkNum, const zbal_tensor_info_t *topkIndex,
                               const zbal_tensor_info_t *topkWeight, aclrtStream stream, int64_t flags) = 0;
     virtual int32_t WeightPrepack(const zbal_tensor_info_t *src, const zbal_tensor_info_t *dst, aclrtStream stream,

@@ -56,7 +56,7 @@ public:
                          const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                          const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                          const zbal_tensor_info_t *, const zbal_tensor_info_t *, const zbal_tensor_info_t *, int64_t,
-                         int64_t, int64_t, int64_t, int64_t, aclrtStream, int64_t) override { return Z_OK; }
+                         int64_t, int64_t, int64_t, int64_t, bool, aclrtStream, int64_t) override { return Z_OK; }
     int32_t TopkRoute(const zbal_tensor_info_t *, int64_t, const zbal_tensor_info_t *, const zbal_tensor_info_t *,
                       aclrtStream, int64_t) override { return Z_OK; }
     int32_t WeightPrepack(const zbal_tensor_info_t *, const zbal_tensor_info_t *, aclrtStream, int64_t) override { return Z_OK; }

@@ -52,11 +52,26 @@ struct GemmParams {
     int K;
     int N;                   /* weight rows per expert (N1 for GMM1) */
     int wscale_is_bf16;
+    int w_is_list;           /* `w` and `wscale` are device tables of `experts` addresses, one expert's tensor each */
     void *out;               /* GMM1: q2 bytes; GMM2: y */
     float *out_scale;        /* GMM1: scale2 (fp8 mode) */
     float *sgl_ws;           /* GMM1 int8 modes: fp32 SwiGLU values [rows, N/2] */
     uint32_t *rowmax;        /* GMM1 int8 modes: per-row absmax bits */
 };
+
+/*
+ * First element of expert e's weights or scales: base + e * stride, or entry e of the address table. The table is
+ * read through the constant address space: a scalar load, which does not queue behind the slabs in flight.
+ */
+template <typename T>
+__device__ __forceinline__ const T *expert_base(const void *base, int is_list, int expert, int64_t stride_elems)
+{
+    if (is_list) {
+        typedef const uint64_t __attribute__((address_space(4))) *table_t;
+        return (const T *)(uintptr_t)((table_t)(uintptr_t)base)[expert];
+    }
+    return (const T *)base + (int64_t)expert * stride_elems;
+}
 
 struct TileCoord {
     int expert, m_tile, n_tile;
@@ -103,11 +118,11 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
                 if constexpr (MODE == MODE_W8A8) {
                     float ws[4];
                     if (p.wscale_is_bf16) {
-                        const u32x2 v = *reinterpret_cast<const u32x2 *>((const uint16_t *)p.wscale + (int64_t)tc.expert * p.N + n);
+                        const u32x2 v = *reinterpret_cast<const u32x2 *>(expert_base<uint16_t>(p.wscale, p.w_is_list, tc.expert, p.N) + n);
                         ws[0] = zb_bf16_to_f32(v[0] & 0xffffu); ws[1] = zb_bf16_to_f32(v[0] >> 16);
                         ws[2] = zb_bf16_to_f32(v[1] & 0xffffu); ws[3] = zb_bf16_to_f32(v[1] >> 16);
                     } else {
-                        const f32x4 v = *reinterpret_cast<const f32x4 *>((const float *)p.wscale + (int64_t)tc.expert * p.N + n);
+                        const f32x4 v = *reinterpret_cast<const f32x4 *>(expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N) + n);
                         ws[0] = v[0]; ws[1] = v[1]; ws[2] = v[2]; ws[3] = v[3];
                     }
 #pragma unroll
@@ -142,7 +157,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
                 const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
                 float g[4], u[4];
                 if constexpr (MODE == MODE_W8A8) {
-                    const float *wsb = (const float *)p.wscale + (int64_t)tc.expert * p.N;
+                    const float *wsb = expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N);
                     const f32x4 wg = *reinterpret_cast<const f32x4 *>(wsb + j);
                     const f32x4 wu = *reinterpret_cast<const f32x4 *>(wsb + I + j);
 #pragma unroll
@@ -412,10 +427,11 @@ grouped_gemm_dma_kernel(GemmParams p)
         t.sa_base = p.a_scale + (int64_t)t.row_begin * KB;
         /* weights come pre-packed as 16 KiB blocks of 128 channels x 128 K-bytes in LDS order ([E][N/128][K/128]) */
         const int col0 = GMM1 ? t.n_tile : t.n_tile * 2, col1 = GMM1 ? I / 128 + t.n_tile : t.n_tile * 2 + 1;
-        t.w_half[0] = p.w + (((int64_t)expert * (p.N / 128) + col0) * KB) * W_BLOCK_BYTES;
-        t.w_half[1] = p.w + (((int64_t)expert * (p.N / 128) + col1) * KB) * W_BLOCK_BYTES;
+        const uint8_t *wb = expert_base<uint8_t>(p.w, p.w_is_list, expert, (int64_t)(p.N / 128) * KB * W_BLOCK_BYTES);
+        t.w_half[0] = wb + ((int64_t)col0 * KB) * W_BLOCK_BYTES;
+        t.w_half[1] = wb + ((int64_t)col1 * KB) * W_BLOCK_BYTES;
         if (MODE == MODE_W4A8) {      /* fp16 group scales [E][K/128][N]: the slab's 128 scales of each half are 256 bytes */
-            const uint16_t *gs = (const uint16_t *)p.wscale + (int64_t)expert * KB * p.N;
+            const uint16_t *gs = expert_base<uint16_t>(p.wscale, p.w_is_list, expert, (int64_t)KB * p.N);
             t.gs_mine = gs + ((wave_u & 1) ? col1 : col0) * 128;
         }
     };
@@ -467,7 +483,7 @@ grouped_gemm_dma_kernel(GemmParams p)
     auto issue_sw = [&](const Tile &t, int buf) __attribute__((always_inline)) {
         if (MODE != MODE_FP8) return;
         const int sw_stride = p.N / 128;
-        const float *base = (const float *)p.wscale + (int64_t)t.expert * KB * sw_stride;
+        const float *base = expert_base<float>(p.wscale, p.w_is_list, t.expert, (int64_t)KB * sw_stride);
         const int c0 = GMM1 ? t.n_tile : t.n_tile * 2, c1 = GMM1 ? I / 128 + t.n_tile : t.n_tile * 2 + 1;
         for (int b = wave_u * 64; b < KB; b += NW * 64) {
             if (b + lane < KB) {
@@ -768,6 +784,8 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
                                              int64_t n1, int32_t mode, void *q2, float *scale2, float *sgl_ws,
                                              void *stream)
 {
+    const int w_is_list = (mode & ZBALHIP_WEIGHTS_AS_LISTS) != 0;
+    mode &= ~ZBALHIP_WEIGHTS_AS_LISTS;
     if (!a || !a_scale || !w1 || !w1scale || !row_off || !q2 || !scale2) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
     if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || k > 128 * 256 || n1 <= 0 || n1 % 256 != 0)
@@ -777,7 +795,7 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
     GemmParams p = {};
     p.a = (const uint8_t *)a; p.a_scale = a_scale; p.w = (const uint8_t *)w1; p.wscale = w1scale; p.row_off = row_off;
     p.experts = (int)experts; p.max_rows = (int)max_rows; p.K = (int)k; p.N = (int)n1;
-    p.out = q2; p.out_scale = scale2; p.sgl_ws = sgl_ws;
+    p.out = q2; p.out_scale = scale2; p.sgl_ws = sgl_ws; p.w_is_list = w_is_list;
     const int n_tiles = (int)(n1 / 2 / 128);
     if (mode == MODE_FP8) return launch_dma<MODE_FP8, true, ZDT_BF16>(p, n_tiles, st);
     if (!sgl_ws) return ZBALHIP_INVALID;
@@ -802,6 +820,8 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
                                         int64_t max_rows, int64_t k, int64_t n, int32_t mode, int32_t out_dtype,
                                         void *y, void *stream)
 {
+    const int w_is_list = (mode & ZBALHIP_WEIGHTS_AS_LISTS) != 0;
+    mode &= ~ZBALHIP_WEIGHTS_AS_LISTS;
     if (!a || !a_scale || !w2 || !wscale || !row_off || !y) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
     if (out_dtype != ZDT_BF16 && out_dtype != ZDT_FP16) return ZBALHIP_INVALID;
@@ -814,6 +834,7 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
     p.a = (const uint8_t *)a; p.a_scale = a_scale; p.w = (const uint8_t *)w2; p.wscale = wscale; p.row_off = row_off;
     p.experts = (int)experts; p.max_rows = (int)max_rows; p.K = (int)k; p.N = (int)n;
     p.wscale_is_bf16 = (wscale_dtype == ZDT_BF16);
+    p.w_is_list = w_is_list;
     p.out = y;
     const int n_tiles = (int)(n / BN);
     const bool bf = out_dtype == ZDT_BF16;

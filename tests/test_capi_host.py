@@ -183,7 +183,7 @@ def test_operator_validation_codes(host_world):
     assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 256, 0, 0, world, None, 0) == 0
     assert lib.zbal_fused_deep_moe(*fused, 0, 0, 0, 256, 0, 0, world, None, 0) == -2
     assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 0, 0, 0, world, None, 0) == -2
-    assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 256, 0, 1, world, None, 0) == -2              # tensor list
+    assert lib.zbal_fused_deep_moe(*fused, 8, 0, 0, 256, 0, 1, world, None, 0) == 0               # tensor list
     half = list(fused); half[8] = ctypes.byref(capi.TensorInfo(data=ctypes.c_void_p(0x1000)))  # shared gmm1 weight alone
     assert lib.zbal_fused_deep_moe(*half, 8, 0, 0, 256, 256, 0, world, None, 0) == -2
     bad = list(fused); bad[17] = None

@@ -417,6 +417,40 @@ def test_fused_moe_active_mask(buf, mode, active):
         assert np.array_equal(got[:active], ref)
 
 
+@pytest.mark.parametrize("mode", [0, 2, 3])
+@pytest.mark.parametrize("T", [70, 700])
+def test_fused_moe_tensor_list_weights(buf, mode, T):
+    """Tensor-list weights (EXEC_FLAG_TENSOR_LIST, ...swiglu_quant_multistage_workspace.h:669-673, 755-757, 1531-1558):
+    every expert's weights and scales are separate allocations, found through a table of addresses. Same arithmetic,
+    so the result must equal the stacked call bit for bit (and the oracle to the mode's bar)."""
+    H, K, E, I = 256, 4, 8, 128
+    x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 140 + mode)
+    int4 = mode == 3
+    sdt1 = torch.float16 if mode == 3 else None
+    sdt2 = {0: torch.bfloat16, 2: None, 3: torch.float16}[mode]
+    xd, idd, esd = dev(x, torch.bfloat16), dev(ids), dev(es)
+    stacked, _, nums_s = buf.fused_deep_moe(xd, idd, buf.prepack_weight(dev(w1), int4=int4), dev(s1, sdt1),
+                                            buf.prepack_weight(dev(w2), int4=int4), dev(s2, sdt2), esd, E, quant_mode=mode)
+    pad = []                                             # allocations in between, so that the experts are not adjacent
+    def each(a, dt=None, pack=False):
+        out = []
+        for e in range(E):
+            t = dev(a[e:e + 1], dt)
+            out.append(buf.prepack_weight(t, int4=int4) if pack else t.clone())
+            pad.append(torch.empty(4096 * (e + 1), device="cuda", dtype=torch.uint8))
+        return out
+    lists = each(w1, pack=True), each(s1, sdt1), each(w2, pack=True), each(s2, sdt2)
+    out, _, nums = buf.fused_deep_moe(xd, idd, *lists, esd, E, quant_mode=mode, is_tensor_list=True)
+    assert np.array_equal(host(nums), host(nums_s))
+    assert np.array_equal(host(out), host(stacked))
+    ref, counts = zo.fused_moe(x, zo.DT_BF16, ids, es, w1, s1, w2, s2, E, mode)
+    assert np.array_equal(host(nums), counts)
+    if mode == 2:
+        assert max_rel_err(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(ref)) < 2e-2
+    else:
+        assert np.array_equal(host(out), ref)
+
+
 def test_fused_moe_empty_experts_and_invalid_ids(buf):
     T, H, K, E, I = 16, 256, 2, 32, 128                  # 32 picks over 32 experts: most experts are empty
     x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, 0, 90, zipf=1.2)
