@@ -77,7 +77,7 @@ combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base,
         }
         u32x4 o;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = zb_f32_to_half<DT>(acc[2 * i]) | (zb_f32_to_half<DT>(acc[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) o[i] = zb_pack2_half<DT>(acc[2 * i], acc[2 * i + 1]);
         __builtin_nontemporal_store(o, reinterpret_cast<u32x4 *>(out + (int64_t)t * hidden + (int64_t)c * 8));
     }
 }

@@ -135,8 +135,8 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
                     for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i] * xs;
                 }
                 u32x2 o;
-                o[0] = zb_f32_to_half<OUT_DT>(d[0]) | (zb_f32_to_half<OUT_DT>(d[1]) << 16);
-                o[1] = zb_f32_to_half<OUT_DT>(d[2]) | (zb_f32_to_half<OUT_DT>(d[3]) << 16);
+                o[0] = zb_pack2_half<OUT_DT>(d[0], d[1]);
+                o[1] = zb_pack2_half<OUT_DT>(d[2], d[3]);
                 *reinterpret_cast<u32x2 *>(y + (int64_t)row * p.N + n) = o;
             }
         }

@@ -75,7 +75,7 @@ template <int DT> __device__ __forceinline__ u32x4 pack(const typename Elem<DT>:
         for (int i = 0; i < 4; ++i) v[i] = __float_as_uint(a[i]);
     } else if constexpr (DT == ZDT_BF16 || DT == ZDT_FP16) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = zb_f32_to_half<DT>(a[2 * i]) | (zb_f32_to_half<DT>(a[2 * i + 1]) << 16);
+        for (int i = 0; i < 4; ++i) v[i] = zb_pack2_half<DT>(a[2 * i], a[2 * i + 1]);
     } else if constexpr (DT == ZDT_INT32) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) v[i] = a[i];

@@ -43,13 +43,15 @@ static inline int32_t zbalhip_check_launch()
 
 __device__ __forceinline__ float zb_bf16_to_f32(uint32_t h) { return __uint_as_float(h << 16); }
 
-__device__ __forceinline__ uint32_t zb_f32_to_bf16(float f)
+/* two floats -> two bf16 in one dword: v_cvt_pk_bf16_f32, round to nearest even, NaN stays a quiet NaN */
+__device__ __forceinline__ uint32_t zb_pack2_bf16(float lo, float hi)
 {
-    uint32_t u = __float_as_uint(f);
-    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f32x2_t{lo, hi}, bf16x2_t));
 }
+
+__device__ __forceinline__ uint32_t zb_f32_to_bf16(float f) { return zb_pack2_bf16(f, 0.0f) & 0xffffu; }
 
 __device__ __forceinline__ float zb_fp16_to_f32(uint32_t h)
 {
@@ -82,6 +84,13 @@ template <int DT> __device__ __forceinline__ uint32_t zb_f32_to_half(float f)
 {
     if constexpr (DT == ZDT_FP16) return zb_f32_to_fp16(f);
     else return zb_f32_to_bf16(f);
+}
+
+/* two values rounded to DT, `lo` in the low half of the dword */
+template <int DT> __device__ __forceinline__ uint32_t zb_pack2_half(float lo, float hi)
+{
+    if constexpr (DT == ZDT_FP16) return zb_f32_to_fp16(lo) | (zb_f32_to_fp16(hi) << 16);
+    else return zb_pack2_bf16(lo, hi);
 }
 
 /* two floats -> two e4m3 codes in the low 16 bits (v_cvt_pk_fp8_f32, OCP format on gfx950); inputs pre-clamped */
