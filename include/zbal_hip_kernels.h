@@ -96,15 +96,45 @@ ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype,
                                      int32_t *scratch, int32_t scratch_blocks, void *stream);
 
 /*
+ * Device trace ring (reference aicore/common/zbal_kernel_trace.h:22-62, layout
+ * constants zbal_comm_host_device_struct.h:22-25). The ring is host memory the
+ * GPU can write: ZBALHIP_TRACE_UNITS blocks of `points` 64-bit words; word
+ * [ZBALHIP_TRACE_IDX_OFF] of a block is the index of its newest record and
+ * records start at [ZBALHIP_TRACE_REC_OFF]. A record is
+ * frame << 56 | end << 62 | timestamp, the timestamp in ticks of the GPU's
+ * constant 100 MHz clock. Workgroup b < ZBALHIP_TRACE_UNITS of a traced kernel
+ * writes to block b (one lane, begin and end of each frame); a block that is
+ * full drops further records.
+ *   zbalhip_trace_alloc: pinned, zeroed host memory and its device address.
+ *   zbalhip_trace_configure: the ring that kernels launched from now on write
+ *     to (null = tracing off, the state at start-up). One ring per process.
+ *   zbalhip_trace_sync: waits until the device is idle, so that the ring holds
+ *     every record of the kernels launched so far.
+ *   zbalhip_trace_free: waits for the device, then releases the memory.
+ */
+#define ZBALHIP_TRACE_UNITS 64
+#define ZBALHIP_TRACE_IDX_OFF 8
+#define ZBALHIP_TRACE_REC_OFF 16
+#define ZBALHIP_TRACE_FRAME_SHIFT 56
+#define ZBALHIP_TRACE_BE_SHIFT 62
+ZBALHIP_API int32_t zbalhip_trace_alloc(int64_t points, uint64_t **host_ring, uint64_t **device_ring);
+ZBALHIP_API int32_t zbalhip_trace_configure(uint64_t *device_ring, int64_t points);
+ZBALHIP_API int32_t zbalhip_trace_sync(void);
+ZBALHIP_API int32_t zbalhip_trace_free(uint64_t *host_ring);
+
+/*
  * The local reduction under ZBALOpReduceScatter / ZBALOpAllReduce
  * (zbal_npu_operators.h:21-25; kernels reducescatter.cpp:94-151,
  * allreduce.cpp:206-260): out[j] = op over p = 0..n_in-1 of in[p][j].
  * `in` is a HOST array of n_in <= ZBALHIP_MAX_REDUCE_PEERS device pointers.
  * Float types accumulate in fp32 in order p = 0..n_in-1 and round once.
- * op is a zbal_reduce_op_t value; PROD is a true product.
+ * op is a zbal_reduce_op_t value; PROD is a true product. trace_frame != 0
+ * (a zbal_profiling_name_t value of the reference,
+ * zbal_comm_host_device_struct.h:27-70) records that frame around each traced
+ * workgroup's work when a trace ring is configured.
  */
 ZBALHIP_API int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t count, int32_t dtype, int32_t op, void *out,
-                       void *stream);
+                       int32_t trace_frame, void *stream);
 
 /* p[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node) */
 ZBALHIP_API int32_t zbalhip_fill_i32(int32_t *p, int64_t n, int32_t value, void *stream);

@@ -37,6 +37,19 @@ void zbal_comm_destroy_all(uint32_t flags);
 int32_t zbal_comm_register_peer_window(zbal_comm_t comm, uint16_t rank, void *base, uint64_t size);
 
 /*
+ * extension: write the communicator's device trace now (the reference does it
+ * when the communicator is destroyed and on SIGUSR1, Communicator::
+ * DumpProfilingTrace zbal_communicator.h:114, zbal_npu_communicator_base.cpp:
+ * 215-276; both still happen here at destruction). Tracing is switched on
+ * with the reference's environment variables, read when a communicator is
+ * created: ZBAL_PROF_ENABLE=1, ZBAL_PROF_MAX_TRACING_COUNT, ZBAL_PROF_DIR.
+ * The file is trace_view_<rank>_<group index>_<date>.json in ZBAL_PROF_DIR, a
+ * trace-viewer (chrome://tracing) array of begin / end events, one "thread"
+ * per traced workgroup. Returns 0, also when tracing is off.
+ */
+int32_t zbal_comm_dump_profiling_trace(zbal_comm_t comm);
+
+/*
  * reference zbal_operations.h:82-83. One-GPU share: recv[j] = reduce over
  * ranks p = 0..R-1 of peer_p(send)[j] for all `count` elements (the
  * reduce-scatter phase of every slice followed by the all-gather, which on

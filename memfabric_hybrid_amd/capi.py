@@ -87,6 +87,7 @@ SIGNATURES = {
     "zbal_comm_destroy": (_i32, [_vp, _u32]),
     "zbal_comm_destroy_all": (None, [_u32]),
     "zbal_comm_register_peer_window": (_i32, [_vp, _u16, _vp, _u64]),
+    "zbal_comm_dump_profiling_trace": (_i32, [_vp]),
     "zbal_all_reduce": (_i32, [_vp, _vp, _vp, ctypes.c_size_t, _i32, _i32, _vp, _vp]),
     "zbal_reduce_scatter": (_i32, [_vp, _vp, ctypes.c_size_t, _i32, _i32, _vp, _vp]),
     "zbal_dispatch_normal_notify": (_i32, [_TI, _i64, _i64, _TI, _TI, _TI, _TI, _TI, _vp, _vp, _i64]),
@@ -108,7 +109,11 @@ SIGNATURES = {
     "zbalhip_combine": (_i32, [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "zbalhip_dispatch_low_latency": (_i32, [_vp, _i32, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp,
                                             _vp, _vp, _i32, _vp]),
-    "zbalhip_reduce": (_i32, [ctypes.POINTER(_vp), _i32, _i64, _i32, _i32, _vp, _vp]),
+    "zbalhip_reduce": (_i32, [ctypes.POINTER(_vp), _i32, _i64, _i32, _i32, _vp, _i32, _vp]),
+    "zbalhip_trace_alloc": (_i32, [_i64, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint64)), ctypes.POINTER(ctypes.POINTER(ctypes.c_uint64))]),
+    "zbalhip_trace_configure": (_i32, [ctypes.POINTER(ctypes.c_uint64), _i64]),
+    "zbalhip_trace_sync": (_i32, []),
+    "zbalhip_trace_free": (_i32, [ctypes.POINTER(ctypes.c_uint64)]),
     "zbalhip_weight_prepack": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp]),
     "zbalhip_fill_i32": (_i32, [_vp, _i64, _i32, _vp]),
     "zbalhip_fused_permute_quant": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp,

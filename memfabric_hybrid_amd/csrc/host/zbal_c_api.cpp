@@ -129,6 +129,14 @@ ZBAL_API int32_t zbal_comm_register_peer_window(zbal_comm_t comm, uint16_t rank,
     return Z_OK;
 }
 
+ZBAL_API int32_t zbal_comm_dump_profiling_trace(zbal_comm_t comm)
+{
+    CommunicatorPtr c = Resolve("DumpProfilingTrace", comm);
+    if (!c) return Z_INVALID_PARAM;
+    c->DumpProfilingTrace();
+    return Z_OK;
+}
+
 /* ---- reductions: reference zbal_operations.cpp:117-157 ------------------------ */
 
 ZBAL_API int32_t zbal_all_reduce(const void *send_buff, void *recv_buff, void *buffer, size_t count,

@@ -10,7 +10,10 @@
  * "peer" output buffers are the caller's local tensors. Reductions run over
  * the group's registered peer windows.
  */
+#include <cstdlib>
 #include <cstring>
+#include <ctime>
+#include <fstream>
 
 #include "zbal_hip_kernels.h"
 #include "zbal_host.h"
@@ -71,9 +74,104 @@ int32_t Launched(const char *op, int32_t rc)
     return rc;
 }
 
+/* names of the frames the kernels record, by zbal_profiling_name_t value (reference
+   zbal_comm_host_device_struct.h:27-70 and g_profName :76-120) */
+enum { PROF_RS_KERNEL_ALL = 7, PROF_AR_KERNEL_ALL = 17 };
+const char *ProfName(uint64_t frame)
+{
+    switch (frame) {
+        case PROF_RS_KERNEL_ALL: return "RS_KERNEL_ALL";
+        case PROF_AR_KERNEL_ALL: return "AR_KERNEL_ALL";
+        default: return nullptr;
+    }
+}
+
 class GpuCommunicator final : public Communicator {
 public:
-    using Communicator::Communicator;
+    /*
+     * Tracing follows the reference's switches (zbal_env_helper.h:20-22, SetupProfMemory
+     * zbal_npu_communicator_base.cpp:145-199): ZBAL_PROF_ENABLE=1 turns it on, ZBAL_PROF_MAX_TRACING_COUNT is the
+     * number of 64-bit words per traced workgroup (20480 unless in [20480, 204800)), ZBAL_PROF_DIR the directory
+     * of the dump. The ring is pinned host memory the kernels write directly. The process has one active ring:
+     * the one of the communicator created last with tracing on.
+     */
+    explicit GpuCommunicator(const GroupInfo &info) : Communicator(info)
+    {
+        const char *sw = std::getenv("ZBAL_PROF_ENABLE");
+        if (sw == nullptr || std::atoi(sw) != 1) return;
+        int64_t points = 20480;
+        if (const char *c = std::getenv("ZBAL_PROF_MAX_TRACING_COUNT")) {
+            const long long v = std::atoll(c);
+            if (v >= 20480 && v < 204800) points = v;
+        }
+        if (zbalhip_trace_alloc(points, &traceHost_, &traceDev_) != 0) {
+            ZBAL_LOG_AND_SET_LAST_ERROR("Failed to allocate " << points * ZBALHIP_TRACE_UNITS * 8 << " bytes of trace memory");
+            traceHost_ = traceDev_ = nullptr;
+            return;
+        }
+        tracePoints_ = points;
+        zbalhip_trace_configure(traceDev_, tracePoints_);
+    }
+
+    ~GpuCommunicator() override
+    {
+        if (traceHost_ == nullptr) return;
+        DumpProfilingTrace();
+        zbalhip_trace_configure(nullptr, 0);
+        zbalhip_trace_free(traceHost_);
+    }
+
+    /*
+     * One begin / end event per record, in the format of the reference's trace-viewer writer
+     * (zbal_trace_viewer_dumper.h:277-304; DumpProfilingTrace zbal_npu_communicator_base.cpp:215-271): a JSON
+     * array that chrome://tracing and Perfetto load. Timestamps are microseconds of the GPU's 100 MHz clock.
+     */
+    void DumpProfilingTrace() noexcept override
+    {
+        if (traceHost_ == nullptr) return;
+        if (zbalhip_trace_sync() != 0) return;
+        const char *dir = std::getenv("ZBAL_PROF_DIR");
+        char stamp[64];
+        std::time_t now = std::time(nullptr);
+        struct tm lt;
+        localtime_r(&now, &lt);
+        std::strftime(stamp, sizeof(stamp), "%Y_%m_%d_%H_%M_%S", &lt);
+        const uint32_t rank = info_.myGroupRank;
+        const std::string path = std::string(dir ? dir : "/home/") + "/trace_view_" + std::to_string(rank) + "_" +
+                                 std::to_string(info_.groupIndex) + "_" + stamp + ".json";
+        std::ofstream f(path);
+        if (!f) {
+            ZBAL_LOG_AND_SET_LAST_ERROR("rank " << rank << " print profiling, open dump file " << path << " failed");
+            return;
+        }
+        f << "[";
+        bool first = true;
+        for (uint64_t u = 0; u < ZBALHIP_TRACE_UNITS; ++u) {
+            const uint64_t *blk = traceHost_ + u * tracePoints_;
+            for (uint64_t j = ZBALHIP_TRACE_REC_OFF; j < (uint64_t)tracePoints_; ++j) {
+                const uint64_t rec = blk[j];
+                const uint64_t frame = (rec >> ZBALHIP_TRACE_FRAME_SHIFT) & ((1u << (ZBALHIP_TRACE_BE_SHIFT - ZBALHIP_TRACE_FRAME_SHIFT)) - 1);
+                if (frame == 0) break; /* the rest of the block is empty */
+                const char *name = ProfName(frame);
+                if (name == nullptr) break;
+                const bool end = (rec >> ZBALHIP_TRACE_BE_SHIFT) & 1;
+                const uint64_t ticks = rec & ((1ull << ZBALHIP_TRACE_FRAME_SHIFT) - 1);
+                char ts[32];
+                std::snprintf(ts, sizeof(ts), "%llu.%02llu", (unsigned long long)(ticks / 100), (unsigned long long)(ticks % 100));
+                f << (first ? "\n" : ",\n") << "{\"name\":\"" << name << "\", \"ph\":\"" << (end ? 'E' : 'B')
+                  << "\", \"pid\":\"RANK_" << rank << "\", \"tid\":\"wg " << u << "\", \"ts\":" << ts << "}";
+                first = false;
+            }
+        }
+        f << "\n]";
+        ZBAL_LOG(LOG_INFO, "dump trace " << info_.groupIndex << " on rank " << rank << " finished: " << path);
+    }
+
+private:
+    uint64_t *traceHost_ = nullptr, *traceDev_ = nullptr;
+    int64_t tracePoints_ = 0;
+
+public:
 
     bool SingleRank(const char *op) const
     {
@@ -114,7 +212,7 @@ public:
         }
     }
 
-    int32_t Reduce(const char *opName, const void *send, size_t sliceOffsetElems, void *recv, size_t count,
+    int32_t Reduce(const char *opName, int traceFrame, const void *send, size_t sliceOffsetElems, void *recv, size_t count,
                    zbal_datatype_t dt, zbal_reduce_op_t op, aclrtStream stream)
     {
         switch (dt) { /* the types the reference instantiates, zbal_kernel_allreduce.cpp:378-416 */
@@ -138,19 +236,20 @@ public:
         }
         for (uint16_t r = 0; r < info_.groupSize; ++r)
             peer[r] = static_cast<const uint8_t *>(peer[r]) + sliceOffsetElems * es;
-        return Launched(opName, zbalhip_reduce(peer, info_.groupSize, (int64_t)count, dt, op, recv, stream));
+        return Launched(opName, zbalhip_reduce(peer, info_.groupSize, (int64_t)count, dt, op, recv, traceFrame, stream));
     }
 
     int32_t AllReduce(const void *send, void *recv, void *, size_t count, zbal_datatype_t dt, zbal_reduce_op_t op,
                       aclrtStream stream) override
     {
-        return Reduce("AllReduce", send, 0, recv, count, dt, op, stream);
+        return Reduce("AllReduce", PROF_AR_KERNEL_ALL, send, 0, recv, count, dt, op, stream);
     }
 
     int32_t ReduceScatter(const void *send, void *recv, size_t recvCount, zbal_datatype_t dt, zbal_reduce_op_t op,
                           aclrtStream stream) override
     {
-        return Reduce("ReduceScatter", send, (size_t)info_.myGroupRank * recvCount, recv, recvCount, dt, op, stream);
+        return Reduce("ReduceScatter", PROF_RS_KERNEL_ALL, send, (size_t)info_.myGroupRank * recvCount, recv, recvCount, dt, op,
+                      stream);
     }
 
     int32_t DispatchNormalLayout(const zbal_tensor_info_t *topkIndex, int64_t tokens, int64_t expertNum,

@@ -116,6 +116,10 @@ public:
     virtual ~Communicator() = default;
 
     const GroupInfo &Info() const { return info_; }
+
+    /* writes what the device trace ring holds as a trace-viewer file; a no-op when tracing is off
+       (reference zbal_communicator.h:114) */
+    virtual void DumpProfilingTrace() noexcept {}
     GroupInfo &MutableInfo() { return info_; }
 
     virtual int32_t AllReduce(const void *send, void *recv, void *buffer, size_t count, zbal_datatype_t dt,

@@ -7,6 +7,8 @@
  * copy-then-atomic-accumulate scheme re-reads and re-writes the output slice
  * once per peer.
  */
+#include <string.h>
+
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
 
@@ -14,7 +16,32 @@ namespace {
 
 struct ReducePtrs {
     const void *p[ZBALHIP_MAX_REDUCE_PEERS];
+    unsigned long long *trace;      /* device trace ring or null */
+    uint32_t trace_points;
+    uint32_t trace_frame;
 };
+
+/* the process's trace ring: what zbalhip_trace_configure set last */
+unsigned long long *g_trace_ring = nullptr;
+uint32_t g_trace_points = 0;
+
+/*
+ * One record into this workgroup's block of the ring (reference ZBAL_PROF_RECORD, zbal_kernel_trace.h:22-42):
+ * bump the block's index word, then write the record there. Called by one lane of workgroups below
+ * ZBALHIP_TRACE_UNITS; the ring is host memory, so the stores are made visible to the host with a system fence.
+ */
+__device__ __forceinline__ void trace_record(const ReducePtrs &in, bool end)
+{
+    if (in.trace == nullptr || in.trace_frame == 0 || blockIdx.x >= ZBALHIP_TRACE_UNITS || threadIdx.x != 0) return;
+    unsigned long long *blk = in.trace + (uint64_t)blockIdx.x * in.trace_points;
+    unsigned long long idx = blk[ZBALHIP_TRACE_IDX_OFF] + 1;
+    if (idx <= ZBALHIP_TRACE_REC_OFF) idx = ZBALHIP_TRACE_REC_OFF;
+    if (idx >= in.trace_points) return;
+    const unsigned long long ts = (unsigned long long)wall_clock64() & ((1ull << ZBALHIP_TRACE_FRAME_SHIFT) - 1);
+    blk[idx] = ((unsigned long long)in.trace_frame << ZBALHIP_TRACE_FRAME_SHIFT) | ((end ? 1ull : 0ull) << ZBALHIP_TRACE_BE_SHIFT) | ts;
+    blk[ZBALHIP_TRACE_IDX_OFF] = idx;
+    __threadfence_system();
+}
 
 enum { OP_PROD = 0, OP_SUM = 1, OP_MAX = 2, OP_MIN = 3 };
 
@@ -122,6 +149,7 @@ reduce_kernel(ReducePtrs in, int n_in, int64_t nvec, u32x4 *__restrict__ out)
     typedef typename Elem<DT>::acc_t A;
     constexpr int PER = Elem<DT>::per;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    trace_record(in, false);
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < nvec; i += stride) {
         u32x4 v[N];
 #pragma unroll
@@ -140,6 +168,7 @@ reduce_kernel(ReducePtrs in, int n_in, int64_t nvec, u32x4 *__restrict__ out)
         }
         out[i] = pack<DT>(acc);      /* inputs are streamed (non-temporal loads); the plain store measured 5% faster than a non-temporal one */
     }
+    trace_record(in, true);
 }
 
 /* elements past the last whole 16-byte vector */
@@ -208,12 +237,49 @@ template <int DT> int32_t dispatch_op(const ReducePtrs &ptrs, int n_in, int64_t 
 
 } // namespace
 
+extern "C" int32_t zbalhip_trace_alloc(int64_t points, uint64_t **host_ring, uint64_t **device_ring)
+{
+    if (points <= ZBALHIP_TRACE_REC_OFF || points > (1 << 24) || !host_ring || !device_ring) return ZBALHIP_INVALID;
+    const size_t bytes = (size_t)points * ZBALHIP_TRACE_UNITS * sizeof(uint64_t);
+    void *h = nullptr, *d = nullptr;
+    if (hipHostMalloc(&h, bytes, hipHostMallocMapped) != hipSuccess) return ZBALHIP_RT_ERROR;
+    memset(h, 0, bytes);
+    if (hipHostGetDevicePointer(&d, h, 0) != hipSuccess) {
+        (void)hipHostFree(h);
+        return ZBALHIP_RT_ERROR;
+    }
+    *host_ring = (uint64_t *)h;
+    *device_ring = (uint64_t *)d;
+    return ZBALHIP_OK;
+}
+
+extern "C" int32_t zbalhip_trace_configure(uint64_t *device_ring, int64_t points)
+{
+    if (device_ring != nullptr && (points <= ZBALHIP_TRACE_REC_OFF || points > (1 << 24))) return ZBALHIP_INVALID;
+    g_trace_ring = (unsigned long long *)device_ring;
+    g_trace_points = device_ring ? (uint32_t)points : 0;
+    return ZBALHIP_OK;
+}
+
+extern "C" int32_t zbalhip_trace_sync(void) { return hipDeviceSynchronize() == hipSuccess ? ZBALHIP_OK : ZBALHIP_RT_ERROR; }
+
+extern "C" int32_t zbalhip_trace_free(uint64_t *host_ring)
+{
+    if (!host_ring) return ZBALHIP_INVALID;
+    if (hipDeviceSynchronize() != hipSuccess) return ZBALHIP_RT_ERROR;
+    return hipHostFree(host_ring) == hipSuccess ? ZBALHIP_OK : ZBALHIP_RT_ERROR;
+}
+
 extern "C" int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t count, int32_t dtype, int32_t op,
-                                  void *out, void *stream)
+                                  void *out, int32_t trace_frame, void *stream)
 {
     if (!in || !out || n_in <= 0 || n_in > ZBALHIP_MAX_REDUCE_PEERS || count <= 0) return ZBALHIP_INVALID;
+    if (trace_frame < 0 || trace_frame >= (1 << (ZBALHIP_TRACE_BE_SHIFT - ZBALHIP_TRACE_FRAME_SHIFT))) return ZBALHIP_INVALID;
     ReducePtrs ptrs;
     for (int p = 0; p < ZBALHIP_MAX_REDUCE_PEERS; ++p) ptrs.p[p] = p < n_in ? in[p] : nullptr;
+    ptrs.trace = trace_frame ? g_trace_ring : nullptr;
+    ptrs.trace_points = g_trace_points;
+    ptrs.trace_frame = (uint32_t)trace_frame;
     /* the vector path needs 16-byte aligned bases */
     bool aligned = ((uintptr_t)out & 15u) == 0;
     for (int p = 0; p < n_in; ++p) {

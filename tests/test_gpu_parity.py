@@ -209,7 +209,7 @@ def test_reduce_kernel_all_types(buf, dt, op):
         d_in = [dev(a, tdt) for a in ins]
         out = torch.empty_like(d_in[0])
         arr = (ctypes.c_void_p * N)(*[t.data_ptr() for t in d_in])
-        assert lib.zbalhip_reduce(arr, N, n, dt, op, out.data_ptr(), capi.stream_ptr()) == 0
+        assert lib.zbalhip_reduce(arr, N, n, dt, op, out.data_ptr(), 0, capi.stream_ptr()) == 0
         ref = zo.reduce(ins, dt, op)
         assert np.array_equal(host(out), ref), (N, n)
 
@@ -225,7 +225,7 @@ def test_reduce_full_size_sampled_windows(buf):
         ins = [torch.randn(n, device="cuda", generator=g).to(tdt) for _ in range(N)]
         out = torch.empty_like(ins[0])
         arr = (ctypes.c_void_p * N)(*[t.data_ptr() for t in ins])
-        assert lib.zbalhip_reduce(arr, N, n, dt, capi.REDUCE_SUM, out.data_ptr(), capi.stream_ptr()) == 0
+        assert lib.zbalhip_reduce(arr, N, n, dt, capi.REDUCE_SUM, out.data_ptr(), 0, capi.stream_ptr()) == 0
         torch.cuda.synchronize()
         w = 1 << 16
         for start in [0, n - w] + [int(v) for v in rng(6).integers(0, n - w, 6)]:
@@ -275,6 +275,61 @@ def test_reduce_scatter_and_all_reduce_over_peer_windows(buf):
     finally:
         torch.cuda.synchronize()
         destroy_group(comm)
+
+
+def test_device_trace_ring_and_trace_viewer_dump(buf, tmp_path, monkeypatch):
+    """Tracing as the reference switches it on (ZBAL_PROF_ENABLE / ZBAL_PROF_MAX_TRACING_COUNT / ZBAL_PROF_DIR,
+    zbal_env_helper.h:20-22): a communicator created with it records a begin and an end per traced workgroup of each
+    reduce launch and writes a trace-viewer JSON array (zbal_trace_viewer_dumper.h:277-304) on request and when it
+    is destroyed. Results must not change."""
+    import glob
+    import json
+    from memfabric_hybrid_amd.buffer import create_group, destroy_group
+    lib = buf.lib
+    monkeypatch.setenv("ZBAL_PROF_ENABLE", "1")
+    monkeypatch.setenv("ZBAL_PROF_DIR", str(tmp_path))
+    R, me, n = 4, 1, 64 * 1024            # 32 workgroups of 256 lanes x 8 bf16: every one of them is traced
+    comm = create_group("traced4", R, me)
+    try:
+        ins = make_reduce_inputs(capi.DT_BF16, R * n, R, 310)
+        wins = [dev(a, torch.bfloat16) for a in ins]
+        recv = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+        for r in range(R):
+            assert lib.zbal_comm_register_peer_window(comm, r, wins[r].data_ptr(), R * n * 2) == 0
+        launches = 3
+        for _ in range(launches):
+            assert lib.zbal_reduce_scatter(wins[me].data_ptr(), recv.data_ptr(), n, capi.DT_BF16, capi.REDUCE_SUM, comm,
+                                           capi.stream_ptr()) == 0
+        full = torch.empty(R * n, dtype=torch.bfloat16, device="cuda")
+        tmp = torch.empty(n, dtype=torch.bfloat16, device="cuda")
+        assert lib.zbal_all_reduce(wins[me].data_ptr(), full.data_ptr(), tmp.data_ptr(), R * n, capi.DT_BF16,
+                                   capi.REDUCE_SUM, comm, capi.stream_ptr()) == 0
+        assert lib.zbal_comm_dump_profiling_trace(comm) == 0
+        assert np.array_equal(host(recv), zo.reduce([a[me * n:(me + 1) * n].copy() for a in ins], capi.DT_BF16, capi.REDUCE_SUM))
+        files = glob.glob(str(tmp_path / "trace_view_1_*.json"))
+        assert len(files) == 1
+        events = json.load(open(files[0]))
+        wgs = n // (256 * 8)
+        rs = [e for e in events if e["name"] == "RS_KERNEL_ALL"]
+        ar = [e for e in events if e["name"] == "AR_KERNEL_ALL"]
+        assert len(rs) == 2 * launches * wgs and len(ar) == 2 * 64          # the all-reduce has 128 workgroups, 64 traced
+        assert {e["pid"] for e in events} == {"RANK_1"} and {e["tid"] for e in rs} == {"wg %d" % i for i in range(wgs)}
+        for tid in {e["tid"] for e in events}:          # per workgroup: B, E, B, E ... with time going forward
+            mine = [e for e in events if e["tid"] == tid]
+            assert [e["ph"] for e in mine] == ["B", "E"] * (len(mine) // 2)
+            ts = [e["ts"] for e in mine]
+            assert all(b <= a for b, a in zip(ts, ts[1:]))
+            assert ts[-1] - ts[0] < 5e6                                        # microseconds: the launches took well under 5 s
+    finally:
+        torch.cuda.synchronize()
+        destroy_group(comm)
+    assert len(glob.glob(str(tmp_path / "trace_view_1_*.json"))) >= 1         # written again at destruction (same second: same name)
+    monkeypatch.delenv("ZBAL_PROF_ENABLE")
+    plain = create_group("untraced", 1, 0)                                     # tracing off: nothing is written
+    try:
+        assert lib.zbal_comm_dump_profiling_trace(plain) == 0
+    finally:
+        destroy_group(plain)
 
 
 # ---- weight pre-pack --------------------------------------------------------------------------------------
