@@ -637,12 +637,22 @@ grouped_gemm_dma_kernel(GemmParams p)
                 return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
             };
             i32x8 af[4];
+            i32x8 wf_first = {};
 #pragma unroll
             for (int mt = 0; mt < 4; ++mt) {
                 const uint8_t *ab = sb + (wm * 64 + mt * 16) * BKB;
                 const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
                 const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
                 af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                if (mt == 0 && MODE != MODE_W4A8) {
+                    /*
+                     * All waves start their fragment reads together after the barrier and the LDS serves them in the
+                     * order asked, so the two fragments of the first MFMA are asked for before the rest (measured:
+                     * 1.5 % of the kernel; forcing the order of all of them is slower).
+                     */
+                    wf_first = load_w(0);
+                    asm volatile("" ::: "memory");
+                }
             }
 
             if constexpr (MODE == MODE_FP8) {
@@ -658,7 +668,7 @@ grouped_gemm_dma_kernel(GemmParams p)
                     s0[mt] = sa * sw0;
                     s1[mt] = sa * sw1;
                 }
-                i32x8 wf = load_w(0);
+                i32x8 wf = wf_first;
                 f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
 #pragma unroll
                 for (int nt = 0; nt < 8; ++nt) {
@@ -727,7 +737,7 @@ grouped_gemm_dma_kernel(GemmParams p)
                 /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
 #pragma unroll
                 for (int nt = 0; nt < 8; ++nt) {
-                    const i32x8 wf = load_w(nt);
+                    const i32x8 wf = nt == 0 ? wf_first : load_w(nt);
                     if (nt < 4 && more) issue_quarter(nt);
                     const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
 #pragma unroll
