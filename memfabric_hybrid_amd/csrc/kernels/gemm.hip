@@ -647,8 +647,9 @@ grouped_gemm_dma_kernel(GemmParams p)
                 if (mt == 0 && MODE != MODE_W4A8) {
                     /*
                      * All waves start their fragment reads together after the barrier and the LDS serves them in the
-                     * order asked, so the two fragments of the first MFMA are asked for before the rest (measured:
-                     * 1.5 % of the kernel; forcing the order of all of them is slower).
+                     * order asked, so the two fragments of the first MFMA are asked for before the rest (measured,
+                     * alternating with the unordered build on one GPU: 1 % of the kernel; forcing the order of all of them
+                     * is slower).
                      */
                     wf_first = load_w(0);
                     asm volatile("" ::: "memory");
