@@ -102,6 +102,37 @@ def test_gmm1_w8a8_bit_exact(buf, E, K, N1, rows):
     assert np.array_equal(host(q2), r_q2)
 
 
+# experts with no rows, with only a short tile, with exactly full tiles, and with short tails of both classes (1..64 and
+# 65..128 rows): the 256-row shape runs the short tails after all other tiles, the longer class first
+TILE_ORDER_COUNTS = np.array([0, 5, 256, 257, 300, 320, 384, 385, 1024, 1030, 130, 64, 0, 512 + 128, 511, 1], dtype=np.int64)
+
+
+@pytest.mark.parametrize("N", [256, 1280])
+def test_gemms_w8a8_tile_order_with_short_tails_bit_exact(buf, N):
+    counts, K = TILE_ORDER_COUNTS, 384
+    E, rows = len(counts), int(counts.sum())
+    assert rows > 128 * E                                     # so that the launcher takes the 256-row shape
+    a = rng(61).integers(-127, 128, (rows, K)).astype(np.int8)
+    xs = rng(62).uniform(0.005, 0.05, rows).astype(np.float32)
+    w = rng(63).integers(-16, 16, (E, K, N)).astype(np.int8)
+    ws = rng(64).uniform(0.0015, 0.0045, (E, N)).astype(np.float32)
+    y = gmm2(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), capi.DT_FP32, counts, K, N, 1)
+    assert np.array_equal(host(y), zo.grouped_gemm_w8a8_dequant(a, xs, w, ws, counts))
+    q2, s2, _ = gmm1(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), counts, K, N, 1)
+    r_q2, r_s2 = zo.gmm1_swiglu_quant_w8a8(a, xs, w, ws, counts)[:2]
+    assert np.array_equal(host(s2).view(np.uint32), r_s2.view(np.uint32))
+    assert np.array_equal(host(q2), r_q2)
+
+
+def test_gemms_fp8_tile_order_with_short_tails(buf):
+    counts, K, N = TILE_ORDER_COUNTS, 256, 512
+    E, rows = len(counts), int(counts.sum())
+    a, sa, w, sw = fp8_operands(E, K, N, rows, 70)
+    y = gmm2(buf, dev(a), dev(sa), buf.prepack_weight(dev(w)), dev(sw), capi.DT_FP32, counts, K, N, 2)
+    ref = zo.gmm2_fp8(a, sa, w, sw, counts)
+    assert max_rel_err(zo.bf16_to_f32(host(y)), zo.bf16_to_f32(ref)) < 2e-2
+
+
 # ---- fp8 block-scaled ------------------------------------------------------------------------------------------
 
 def fp8_operands(E, K, N, rows, seed):
