@@ -170,10 +170,12 @@ typedef struct {
  * tensor into ZBAL_WEIGHT_FORMAT_PREPACKED, the order in which the grouped
  * GEMM streams it (same number of bytes; K and N multiples of 128):
  *   one byte per element: [E][N/128][K/128] blocks of 16 KiB; a block holds
- *     128 channels x 128 K-bytes, channel r at +128*r, and within a channel
+ *     128 channels x 128 K-bytes, block row r at +128*r, and within a row
  *     the 16-byte chunk c of its K-bytes at slot c ^ (r & 7) ^ ((r >> 3) & 1);
- *   INT4X2: the same block order with 8 KiB blocks (128 channels x 128 k,
- *     two values per byte); channel r at +64*r, and within a channel the
+ *     block row r holds the block's channel
+ *     (r & ~31) | ((r & 15) >> 2) << 3 | ((r >> 4) & 1) << 2 | (r & 3);
+ *   INT4X2: the same block and row order with 8 KiB blocks (128 channels x
+ *     128 k, two values per byte); block row r at +64*r, and within a row the
  *     16-byte chunk c (k in [32c, 32c+32)) at slot c ^ ((r >> 2) & 3); in a
  *     chunk, byte b of dword j holds k[8j+b] in the low and k[8j+4+b] in the
  *     high nibble.

@@ -141,13 +141,16 @@ ZBALHIP_API int32_t zbalhip_fill_i32(int32_t *p, int64_t n, int32_t value, void 
 
 /*
  * Weight pre-pack of [E,K,N] (N contiguous). One byte per element:
- * [E][N/128][K/128] blocks of 128 channels x 128 K-bytes, channel r at +128*r
- * with 16-byte chunk c in slot c ^ (r & 7) ^ ((r >> 3) & 1); k and n multiples
- * of 128, pointers 16-byte aligned. to_int4 != 0 packs int8 values in [-8,7]
- * two per byte into [E][N/128][K/128] blocks of 8 KiB (channel r at +64*r,
- * 16-byte chunk c of 32 k in slot c ^ ((r >> 2) & 3), byte b of dword j =
- * k[8j+b] | k[8j+4+b] << 4). The grouped GEMMs below take `w1` / `w2` in this
- * form.
+ * [E][N/128][K/128] blocks of 128 channels x 128 K-bytes, block row r at
+ * +128*r with 16-byte chunk c in slot c ^ (r & 7) ^ ((r >> 3) & 1); k and n
+ * multiples of 128, pointers 16-byte aligned. Block row r holds channel
+ * (r & ~31) | ((r & 15) >> 2) << 3 | ((r >> 4) & 1) << 2 | (r & 3) of the
+ * block: a lane of the GEMM then ends up with eight consecutive channels.
+ * to_int4 != 0 packs int8 values in [-8,7] two per byte into
+ * [E][N/128][K/128] blocks of 8 KiB (block row r, the same channel as above,
+ * at +64*r, 16-byte chunk c of 32 k in slot c ^ ((r >> 2) & 3), byte b of
+ * dword j = k[8j+b] | k[8j+4+b] << 4). The grouped GEMMs below take `w1` /
+ * `w2` in this form.
  */
 ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int64_t k, int64_t n, int32_t to_int4, void *dst,
                                void *stream);
@@ -191,7 +194,9 @@ ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, 
  * each). mode 2 (fp8): a_scale [rows,K/128], w1scale fp32
  * [E,K/128,N1/128]; q2 e4m3, scale2 [rows,N1/256]; sgl_ws unused.
  * mode 3 (W4A8): w1 pre-packed int4x2 (N1*K/2 bytes per expert), w1scale fp16 [E,K/128,N1];
- * outputs as mode 1. max_rows bounds the launch (>= total rows).
+ * outputs as mode 1. max_rows bounds the launch (>= total rows). a, w1,
+ * w1scale, q2 and sgl_ws must be 16-byte aligned (here and for GMM 2: a, w2,
+ * wscale, y), else ZBALHIP_INVALID.
  */
 ZBALHIP_API int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale, const void *w1, const void *w1scale,
                                   const int32_t *row_off, int64_t experts, int64_t max_rows, int64_t k, int64_t n1,

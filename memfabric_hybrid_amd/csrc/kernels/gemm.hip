@@ -8,26 +8,26 @@
  * WEIGHT fragment as the matrix-A input and the ACTIVATION fragment as the
  * matrix-B input, i.e. it computes C^T. With the 16x16 MFMA output layout
  * (lane l holds output column l%16, rows 4*(l/16)+i) every lane then owns ONE
- * token row and FOUR consecutive output channels per instruction: per-token
- * scales are one value per lane, per-channel scales a 16-byte vector, gate/up
- * pairs of the SwiGLU sit in the same lane, and results leave as 4-element
- * vectors.
+ * token row and FOUR consecutive output channels per instruction, and with
+ * the pre-pack's order of the weight rows EIGHT consecutive channels per pair
+ * of instructions: per-token scales are one value per lane, per-channel
+ * scales 16-byte vectors, gate/up pairs of the SwiGLU sit in the same lane,
+ * and results leave as 8-element vectors.
  *
- * Workgroup tile: 128 token rows x 256 output channels x 128 K-bytes, four
- * waves in a 2x2 grid, each wave 64 rows x 128 channels = 4x8 MFMA tiles
- * (128 accumulator registers). For GMM1 the 256 channels are 128 gate
+ * Workgroup tile: 256 (or 128) token rows x 256 output channels x 128 K-bytes
+ * per step, eight (four) waves, each wave 64 rows x 128 channels = 4x8 MFMA
+ * tiles (128 accumulator registers). For GMM1 the 256 channels are 128 gate
  * columns j and the matching 128 up columns I+j, so the SwiGLU product and,
  * in the fp8 mode, the complete 1x128 requantisation happen in registers.
- * A and W tiles are staged in LDS (rows padded by 16 bytes so that the
- * 16-byte fragment reads of 16 consecutive rows fall in distinct banks);
- * the next K-slab is fetched from HBM into registers while the current one
- * is multiplied (two workgroups per CU hide the barriers).
+ * K slabs go from HBM to LDS by DMA, in a swizzled order that the weights are
+ * pre-packed in, one persistent workgroup per CU; the details stand at the
+ * kernel below.
  *
  * Tile schedule: workgroup ids are dealt round-robin to the 8 XCDs by the
- * hardware, so id -> (id % 8) * chunk + id / 8 gives every XCD a contiguous
- * run of logical tiles; logical tiles walk an expert in groups of
- * (all its row tiles) x (8 channel tiles), row tile fastest, so the ~64
- * workgroups resident on an XCD share both their A and their W slabs in
+ * hardware; XCD x takes a contiguous run of the logical tile order and its
+ * workgroups take consecutive tiles of it. Logical tiles walk an expert in
+ * groups of (all its row tiles) x (8 channel tiles), row tile fastest, so
+ * the workgroups resident on an XCD share both their A and their W slabs in
  * that XCD's L2.
  */
 #include "zbal_device.h"
@@ -91,9 +91,10 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 }
 
 /*
- * Shared epilogue. The calling wave holds, for sub-tile (mt, nt), output channels 4*(lane/16)+i of token
- * row wm*64 + mt*16 + lane%16. `lds_rowmax` is [2][tile_rows] floats of scratch for the row maxima of the
- * two channel halves (GMM1 only).
+ * Shared epilogue. The calling wave holds, for sub-tile (mt, nt), block rows nt*16 + 4*(lane/16) + i of its weight
+ * rows, for token row wm*64 + mt*16 + lane%16. The pre-pack put channels 32*(nt/2) + 8*(lane/16) + 4*(nt%2) + i in
+ * those rows (zb_block_row_channel), so the sub-tiles nt = 2s and 2s+1 together are eight consecutive channels.
+ * `lds_rowmax` is [2][tile_rows] floats of scratch for the row maxima of the two channel halves (GMM1 only).
  */
 template <int MODE, bool GMM1, int OUT_DT>
 __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &tc, f32x4 (&accf)[4][8],
@@ -102,7 +103,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
 {
     const int frag_row = lane & 15;
     const int I = p.N / 2;
-    const int sub_n = (lane >> 4) * 4;
+    const int q8 = (lane >> 4) * 8;
     if constexpr (!GMM1) {
         uint16_t *y = (uint16_t *)p.out;
 #pragma unroll
@@ -112,36 +113,42 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
             float xs = 1.0f;
             if (MODE != MODE_FP8) xs = p.a_scale[row];
 #pragma unroll
-            for (int nt = 0; nt < 8; ++nt) {
-                const int n = tc.n_tile * BN + wn * 128 + nt * 16 + sub_n;
-                float d[4];
+            for (int s = 0; s < 4; ++s) {         /* sub-tiles 2s and 2s+1: eight consecutive channels from n */
+                const int n = tc.n_tile * BN + wn * 128 + s * 32 + q8;
+                float ws[8];
                 if constexpr (MODE == MODE_W8A8) {
-                    float ws[4];
                     if (p.wscale_is_bf16) {
-                        const u32x2 v = *reinterpret_cast<const u32x2 *>(expert_base<uint16_t>(p.wscale, p.w_is_list, tc.expert, p.N) + n);
-                        ws[0] = zb_bf16_to_f32(v[0] & 0xffffu); ws[1] = zb_bf16_to_f32(v[0] >> 16);
-                        ws[2] = zb_bf16_to_f32(v[1] & 0xffffu); ws[3] = zb_bf16_to_f32(v[1] >> 16);
+                        const u32x4 v = *reinterpret_cast<const u32x4 *>(expert_base<uint16_t>(p.wscale, p.w_is_list, tc.expert, p.N) + n);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            ws[2 * i] = zb_bf16_to_f32(v[i] & 0xffffu);
+                            ws[2 * i + 1] = zb_bf16_to_f32(v[i] >> 16);
+                        }
                     } else {
-                        const f32x4 v = *reinterpret_cast<const f32x4 *>(expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N) + n);
-                        ws[0] = v[0]; ws[1] = v[1]; ws[2] = v[2]; ws[3] = v[3];
+                        const float *wsp = expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N) + n;
+                        const f32x4 v0 = *reinterpret_cast<const f32x4 *>(wsp), v1 = *reinterpret_cast<const f32x4 *>(wsp + 4);
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) { ws[i] = v0[i]; ws[4 + i] = v1[i]; }
                     }
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) d[i] = ((float)acci[mt][nt][i] * ws[i]) * xs;
-                } else if constexpr (MODE == MODE_FP8) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i];
-                } else {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) d[i] = accf[mt][nt][i] * xs;
                 }
-                u32x2 o;
-                o[0] = zb_pack2_half<OUT_DT>(d[0], d[1]);
-                o[1] = zb_pack2_half<OUT_DT>(d[2], d[3]);
-                *reinterpret_cast<u32x2 *>(y + (int64_t)row * p.N + n) = o;
+                float d[8];
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const int nt = 2 * s + h;
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        if constexpr (MODE == MODE_W8A8) d[4 * h + i] = ((float)acci[mt][nt][i] * ws[4 * h + i]) * xs;
+                        else if constexpr (MODE == MODE_FP8) d[4 * h + i] = accf[mt][nt][i];
+                        else d[4 * h + i] = accf[mt][nt][i] * xs;
+                    }
+                }
+                *reinterpret_cast<u32x4 *>(y + (int64_t)row * p.N + n) =
+                    u32x4{zb_pack2_half<OUT_DT>(d[0], d[1]), zb_pack2_half<OUT_DT>(d[2], d[3]),
+                          zb_pack2_half<OUT_DT>(d[4], d[5]), zb_pack2_half<OUT_DT>(d[6], d[7])};
             }
         }
     } else {
-        /* SwiGLU on gate sub-tile nt and up sub-tile nt+4: columns j = n_tile*128 + wn*64 + nt*16 + sub_n + i */
+        /* SwiGLU on gate sub-tile nt and up sub-tile nt+4: columns j = n_tile*128 + wn*64 + 32*(nt/2) + q8 + 4*(nt%2) + i */
         float sg[4][4][4];
         float rmax[4];
 #pragma unroll
@@ -154,7 +161,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
             rmax[mt] = 0.0f;
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
-                const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                const int j = tc.n_tile * 128 + wn * 64 + (nt >> 1) * 32 + q8 + (nt & 1) * 4;
                 float g[4], u[4];
                 if constexpr (MODE == MODE_W8A8) {
                     const float *wsb = expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N);
@@ -203,17 +210,20 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
                 const float mult = 448.0f / amax;
                 uint8_t *q2 = (uint8_t *)p.out;
 #pragma unroll
-                for (int nt = 0; nt < 4; ++nt) {
-                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
-                    const uint32_t v = pack4_e4m3(sg[mt][nt][0] * mult, sg[mt][nt][1] * mult, sg[mt][nt][2] * mult,
-                                                  sg[mt][nt][3] * mult);
-                    *reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I + j) = v;
+                for (int s = 0; s < 2; ++s) {         /* sub-tiles 2s and 2s+1: eight consecutive columns */
+                    const int j = tc.n_tile * 128 + wn * 64 + s * 32 + q8;
+                    u32x2 v;
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        v[h] = pack4_e4m3(sg[mt][2 * s + h][0] * mult, sg[mt][2 * s + h][1] * mult, sg[mt][2 * s + h][2] * mult,
+                                          sg[mt][2 * s + h][3] * mult);
+                    *reinterpret_cast<u32x2 *>(q2 + (int64_t)row * I + j) = v;
                 }
                 if (wn == 0 && lane < 16) p.out_scale[(int64_t)row * (I / 128) + tc.n_tile] = amax * (1.0f / 448.0f);
             } else {
 #pragma unroll
                 for (int nt = 0; nt < 4; ++nt) {
-                    const int j = tc.n_tile * 128 + wn * 64 + nt * 16 + sub_n;
+                    const int j = tc.n_tile * 128 + wn * 64 + (nt >> 1) * 32 + q8 + (nt & 1) * 4;
                     const f32x4 v = f32x4{sg[mt][nt][0], sg[mt][nt][1], sg[mt][nt][2], sg[mt][nt][3]};
                     *reinterpret_cast<f32x4 *>(p.sgl_ws + (int64_t)row * I + j) = v;
                 }
@@ -567,9 +577,9 @@ grouped_gemm_dma_kernel(GemmParams p)
         if (GMM1) r = (nt < 4) ? wn * 64 + nt * 16 : 128 + wn * 64 + (nt - 4) * 16;
         else r = wn * 128 + nt * 16;
         w_sub[nt] = A_BYTES + r * WRB;
-        w_ch[nt] = r;                             /* tile-local index of the sub-tile's first output channel */
+        w_ch[nt] = zb_block_row_channel(r);       /* tile-local channel held by the sub-tile's first block row */
     }
-    const int lane_ch = (lane >> 4) * 4;          /* the lane's four channels within a sub-tile */
+    const int lane_ch = (lane >> 4) * 8;          /* block rows 4q .. 4q+3 of a sub-tile hold channels 8q .. 8q+3 past that */
 
     Tile cur, nxt;
     load_tile(lid, cur);
@@ -798,6 +808,9 @@ __global__ void fill_u32_kernel(uint32_t *p, int64_t n, uint32_t v)
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = v;
 }
 
+/* rows, weight blocks and channel scales move as 16-byte vectors (with tensor lists: the tables; their entries are the caller's) */
+inline bool misaligned16(const void *p) { return ((uintptr_t)p & 15) != 0; }
+
 inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles, int tile_m)
 {
     int64_t m_tiles = (max_rows + tile_m - 1) / tile_m + experts;   /* each expert adds at most one partial tile */
@@ -855,6 +868,7 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
     mode &= ~ZBALHIP_WEIGHTS_AS_LISTS;
     if (!a || !a_scale || !w1 || !w1scale || !row_off || !q2 || !scale2) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
+    if (misaligned16(a) || misaligned16(w1) || misaligned16(w1scale) || misaligned16(q2) || misaligned16(sgl_ws)) return ZBALHIP_INVALID;
     if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || k > 128 * 256 || n1 <= 0 || n1 % 256 != 0)
         return ZBALHIP_INVALID;
     if (max_rows == 0) return ZBALHIP_OK;
@@ -891,6 +905,7 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
     mode &= ~ZBALHIP_WEIGHTS_AS_LISTS;
     if (!a || !a_scale || !w2 || !wscale || !row_off || !y) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
+    if (misaligned16(a) || misaligned16(w2) || misaligned16(wscale) || misaligned16(y)) return ZBALHIP_INVALID;
     if (out_dtype != ZDT_BF16 && out_dtype != ZDT_FP16) return ZBALHIP_INVALID;
     if (experts <= 0 || experts > 1024 || max_rows < 0 || k <= 0 || k % 128 != 0 || k > 128 * 256 || n <= 0 || n % BN != 0)
         return ZBALHIP_INVALID;

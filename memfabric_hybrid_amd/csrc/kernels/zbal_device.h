@@ -168,4 +168,15 @@ __device__ __forceinline__ float zb_block_max(float v, float *red)
     return r;
 }
 
+/*
+ * Pre-packed weight blocks: which channel of a 128-channel block sits in block row r. Rows 16t .. 16t+15 feed one
+ * MFMA of the grouped GEMM and rows 4q .. 4q+3 of it come out in the lanes 16q .. 16q+15; the permutation (within
+ * groups of 32 rows) gives those lanes channels 8q .. 8q+3 of the group from the even operand t and 8q+4 .. 8q+7
+ * from the odd one, eight consecutive channels per lane.
+ */
+__host__ __device__ __forceinline__ constexpr int zb_block_row_channel(int r)
+{
+    return (r & ~31) | (((r & 15) >> 2) << 3) | (((r >> 4) & 1) << 2) | (r & 3);
+}
+
 #endif /* ZBAL_DEVICE_H_ */

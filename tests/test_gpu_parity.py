@@ -338,16 +338,21 @@ def test_weight_prepack(buf):
     E, K, N = 3, 256, 384
     w = rng(40).integers(-128, 128, (E, K, N)).astype(np.int8)
     packed = host(buf.prepack_weight(dev(w))).reshape(E, N // 128, K // 128, 128, 8, 16)
-    # block [e][nb][kb] holds channel r at +128*r, 16-byte chunk c of its K-bytes in slot c ^ (r & 7) ^ ((r >> 3) & 1)
-    wt = w.transpose(0, 2, 1).reshape(E, N // 128, 128, K // 128, 8, 16).transpose(0, 1, 3, 2, 4, 5)   # [e][nb][kb][r][c][16]
+    # block [e][nb][kb] holds block row r at +128*r, 16-byte chunk c of its K-bytes in slot c ^ (r & 7) ^ ((r >> 3) & 1);
+    # block row r is channel ch[r] of the block (a permutation within groups of 32)
+    wt = w.transpose(0, 2, 1).reshape(E, N // 128, 128, K // 128, 8, 16).transpose(0, 1, 3, 2, 4, 5)   # [e][nb][kb][ch][c][16]
     r = np.arange(128)
+    ch = (r & ~31) | (((r & 15) >> 2) << 3) | (((r >> 4) & 1) << 2) | (r & 3)
+    assert sorted(ch) == list(range(128)) and np.array_equal(ch[:36], [0, 1, 2, 3, 8, 9, 10, 11, 16, 17, 18, 19, 24, 25, 26, 27,
+                                                                       4, 5, 6, 7, 12, 13, 14, 15, 20, 21, 22, 23, 28, 29, 30, 31,
+                                                                       32, 33, 34, 35])
     f = (r & 7) ^ ((r >> 3) & 1)
     want = np.empty_like(wt)
     for slot in range(8):
-        want[:, :, :, r, slot, :] = wt[:, :, :, r, slot ^ f, :]
+        want[:, :, :, r, slot, :] = wt[:, :, :, ch, slot ^ f, :]
     assert np.array_equal(packed, want)
     assert buf.lib.zbalhip_weight_prepack(dev(w).data_ptr(), E, 200, 136, 0, dev(w).data_ptr() + 16, None) != 0
-    # int4: 8 KiB blocks of 128 channels x 128 k; channel r at +64*r, the 16-byte chunk c (k in [32c, 32c+32)) in slot
+    # int4: 8 KiB blocks of 128 channels x 128 k; block row r (channel ch[r]) at +64*r, the 16-byte chunk c (k in [32c, 32c+32)) in slot
     # c ^ ((r >> 2) & 3) (r taken within its 16-channel group); byte b of dword j = k[8j+b] | k[8j+4+b] << 4
     w4 = rng(41).integers(-8, 8, (E, K, N)).astype(np.int8)
     p4 = host(buf.prepack_weight(dev(w4), int4=True)).reshape(E, N // 128, K // 128, 128, 4, 16)
@@ -357,5 +362,5 @@ def test_weight_prepack(buf):
     f4 = ((r & 15) >> 2) & 3
     want4 = np.empty_like(nib)
     for slot in range(4):
-        want4[:, :, :, r, slot, :] = nib[:, :, :, r, slot ^ f4, :]
+        want4[:, :, :, r, slot, :] = nib[:, :, :, ch, slot ^ f4, :]
     assert np.array_equal(p4, want4)
