@@ -289,8 +289,11 @@ layout_scan_kernel(const int32_t *__restrict__ hist, int nblk, int experts, int 
 
 /* ---- router ----------------------------------------------------------------- */
 
-#define ZB_ROUTE_PER_LANE (ZB_MAX_EXPERTS / 64)
-
+/*
+ * One wave per token; lane l holds logits l, l + 64, ... (PER_LANE of them: the launcher picks the smallest
+ * instantiation that covers `experts`, the arithmetic and its order are the same in all of them).
+ */
+template <int PER_LANE>
 __global__ void __launch_bounds__(256)
 topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int topk, int64_t *__restrict__ topk_idx,
                   float *__restrict__ topk_w)
@@ -299,10 +302,10 @@ topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int
     const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
     if (t >= tokens) return; /* whole waves leave together */
     const float *l = logits + (int64_t)t * experts;
-    float v[ZB_ROUTE_PER_LANE];
+    float v[PER_LANE];
     float mx = -__builtin_inff();
 #pragma unroll
-    for (int j = 0; j < ZB_ROUTE_PER_LANE; ++j) {
+    for (int j = 0; j < PER_LANE; ++j) {
         const int e = j * 64 + lane;
         v[j] = (e < experts) ? l[e] : -__builtin_inff();
         mx = fmaxf(mx, v[j]);
@@ -310,7 +313,7 @@ topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int
     mx = zb_wave_max(mx);
     float sum = 0.0f;
 #pragma unroll
-    for (int j = 0; j < ZB_ROUTE_PER_LANE; ++j) {
+    for (int j = 0; j < PER_LANE; ++j) {
         const int e = j * 64 + lane;
         if (e < experts) sum += zb_expf(v[j] - mx);
     }
@@ -325,7 +328,7 @@ topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int
         float best = -__builtin_inff();
         int bidx = 0x7fffffff;
 #pragma unroll
-        for (int j = 0; j < ZB_ROUTE_PER_LANE; ++j) {
+        for (int j = 0; j < PER_LANE; ++j) {
             const int e = j * 64 + lane;
             if (e < experts && !((used >> j) & 1u)) {
                 if (bidx == 0x7fffffff || v[j] > best) { best = v[j]; bidx = e; }
@@ -439,8 +442,11 @@ extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64
     if (tokens == 0) return ZBALHIP_OK;
     const int wpb = 4;
     const int64_t blocks = (tokens + wpb - 1) / wpb;
-    topk_route_kernel<<<(unsigned)blocks, wpb * 64, 0, (hipStream_t)stream>>>(logits, (int)tokens, (int)experts,
-                                                                           (int)topk, topk_idx, topk_w);
+    const dim3 grid((unsigned)blocks), block(wpb * 64);
+    hipStream_t st = (hipStream_t)stream;
+    if (experts <= 64) topk_route_kernel<1><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, topk_w);
+    else if (experts <= 256) topk_route_kernel<4><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, topk_w);
+    else topk_route_kernel<ZB_MAX_EXPERTS / 64><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, topk_w);
     return zbalhip_check_launch();
 }
 
