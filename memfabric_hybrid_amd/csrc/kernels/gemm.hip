@@ -30,6 +30,8 @@
  * the workgroups resident on an XCD share both their A and their W slabs in
  * that XCD's L2.
  */
+#include <type_traits>
+
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
 
@@ -92,11 +94,12 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 
 /*
  * Shared epilogue. The calling wave holds, for sub-tile (mt, nt), block rows nt*16 + 4*(lane/16) + i of its weight
- * rows, for token row wm*64 + mt*16 + lane%16. The pre-pack put channels 32*(nt/2) + 8*(lane/16) + 4*(nt%2) + i in
+ * rows, for token row (RG*mt + wm)*16 + lane%16 of the tile (RG = row groups of waves; a wave's 16-row sub-tiles
+ * are dealt round-robin over the row groups, so a tile that is not full leaves every SIMD the same share). The pre-pack put channels 32*(nt/2) + 8*(lane/16) + 4*(nt%2) + i in
  * those rows (zb_block_row_channel), so the sub-tiles nt = 2s and 2s+1 together are eight consecutive channels.
  * `lds_rowmax` is [2][tile_rows] floats of scratch for the row maxima of the two channel halves (GMM1 only).
  */
-template <int MODE, bool GMM1, int OUT_DT>
+template <int MODE, bool GMM1, int OUT_DT, int RG>
 __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &tc, f32x4 (&accf)[4][8],
                                          i32x4 (&acci)[4][8], int row_begin, int row_end, int wm, int wn, int lane,
                                          float *lds_rowmax, int tile_rows)
@@ -108,7 +111,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
         uint16_t *y = (uint16_t *)p.out;
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
-            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
+            const int row = row_begin + (RG * mt + wm) * 16 + frag_row;
             if (row >= row_end) continue;
             float xs = 1.0f;
             if (MODE != MODE_FP8) xs = p.a_scale[row];
@@ -153,7 +156,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
         float rmax[4];
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
-            const int row = row_begin + wm * 64 + mt * 16 + frag_row;
+            const int row = row_begin + (RG * mt + wm) * 16 + frag_row;
             int lrow = row;
             if (lrow > p.max_rows - 1) lrow = p.max_rows - 1;
             float xs = 1.0f;
@@ -196,12 +199,12 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
             /* the four lane groups (lane/16) hold different columns of the same row */
             rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 16, 64));
             rmax[mt] = fmaxf(rmax[mt], __shfl_xor(rmax[mt], 32, 64));
-            if (lane < 16) lds_rowmax[wn * tile_rows + wm * 64 + mt * 16 + lane] = rmax[mt];
+            if (lane < 16) lds_rowmax[wn * tile_rows + (RG * mt + wm) * 16 + lane] = rmax[mt];
         }
         __syncthreads();
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
-            const int lr = wm * 64 + mt * 16 + frag_row;
+            const int lr = (RG * mt + wm) * 16 + frag_row;
             const int row = row_begin + lr;
             const float amax_tile = fmaxf(lds_rowmax[lr], lds_rowmax[tile_rows + lr]);
             if (row >= row_end) continue;
@@ -346,7 +349,7 @@ grouped_gemm_dma_kernel(GemmParams p)
     using S = DmaShape<TM, NSTAGE, WRB>;
     constexpr int NW = S::NW, STAGE_BYTES = S::STAGE_BYTES, A_BYTES = S::A_BYTES, W_PARTS = S::W_PARTS, PARTS = S::PARTS;
     constexpr int HALF_BLOCKS = S::HALF_BLOCKS, W_BLOCK_BYTES = 128 * WRB;     /* one 128-channel block of one slab */
-    constexpr bool SKIP_ROW_GROUPS = TM < 256;      /* few-row shape: leave out the MFMAs of absent 16-row groups */
+    constexpr int RG = S::ROW_GROUPS;                /* row groups of waves; 16-row sub-tile s of a tile belongs to group s % RG */
     using Tile = DmaTile;
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     float *lds_sa = reinterpret_cast<float *>(smem + NSTAGE * STAGE_BYTES);   /* [NSTAGE][TM] */
@@ -603,12 +606,18 @@ grouped_gemm_dma_kernel(GemmParams p)
                 accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
                 acci[mt][nt] = i32x4{0, 0, 0, 0};
             }
-        /* a wave whose 64 rows lie past the expert's last row still moves data and meets the barriers, but skips the math */
-        const int rows_here = cur.row_end - (cur.row_begin + wm * 64);
-        const bool wave_active = rows_here > 0;
-        const int mt_act = rows_here >= 64 ? 4 : (rows_here + 15) >> 4;      /* 16-row groups that hold rows */
+        /*
+         * The wave's 16-row sub-tiles are rows (RG*mt + wm)*16 .. +15 of the tile, mt = 0..3. Only the first `mt_act` of
+         * them hold rows of this tile; a wave with none still moves data and meets the barriers, but skips the math.
+         */
+        const int tile_subs = (cur.row_end - cur.row_begin + 15) >> 4;
+        int mt_act = (tile_subs - wm + RG - 1) / RG;
+        mt_act = mt_act < 0 ? 0 : (mt_act > 4 ? 4 : mt_act);
         const float *sw_cur = lds_sw + sw_buf * 2 * D_MAX_KB;
 
+        /* the K loop over the wave's first MT row sub-tiles; MT is a compile-time constant so that the loops unroll */
+        auto k_loop = [&](auto mt_tag) __attribute__((always_inline)) {
+        constexpr int MT = decltype(mt_tag)::value;
         for (int kb = 0; kb < KB; ++kb) {
             /* the slab after this one exists if the tile or the sequence goes on; its loads may stay in flight */
             const bool later = kb + 1 < KB || nxt.valid;
@@ -632,7 +641,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             const uint8_t *sb = smem + stage * STAGE_BYTES;
             const int cur_stage = stage;
             stage = stage + 1 == NSTAGE ? 0 : stage + 1;
-            if (!wave_active) {
+            if constexpr (MT == 0) {
                 if (more) issue(ft, fill_kb, fill_stage);
                 continue;
             }
@@ -640,130 +649,137 @@ grouped_gemm_dma_kernel(GemmParams p)
 #pragma unroll
                 for (int j = q * (PARTS / 4); j < (q + 1) * (PARTS / 4); ++j) issue_part(ft, fill_kb, fill_stage, j);
             };
-
             auto load_w = [&](int nt) -> i32x8 {
                 const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
                 const u32x4 hi = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_hi);
                 return i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
             };
-            i32x8 af[4];
-            i32x8 wf_first = {};
-#pragma unroll
-            for (int mt = 0; mt < 4; ++mt) {
-                const uint8_t *ab = sb + (wm * 64 + mt * 16) * BKB;
-                const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
-                const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
-                af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
-                if (mt == 0 && MODE != MODE_W4A8) {
-                    /*
-                     * All waves start their fragment reads together after the barrier and the LDS serves them in the
-                     * order asked, so the two fragments of the first MFMA are asked for before the rest (measured,
-                     * alternating with the unordered build on one GPU: 1 % of the kernel; forcing the order of all of them
-                     * is slower).
-                     */
-                    wf_first = load_w(0);
-                    asm volatile("" ::: "memory");
-                }
-            }
 
-            if constexpr (MODE == MODE_FP8) {
-                /*
-                 * Software pipeline over the 32 (channel sub-tile, row sub-tile) pairs: the MFMA of pair p+1 is issued
-                 * before the four scale-and-accumulate FMAs of pair p, so the vector ALU works under the matrix unit.
-                 */
-                const float sw0 = sw_cur[kb], sw1 = sw_cur[D_MAX_KB + kb];
-                float s0[4], s1[4];
+            if constexpr (MT > 0) {
+                i32x8 af[MT];
+                i32x8 wf_first = {};
 #pragma unroll
-                for (int mt = 0; mt < 4; ++mt) {
-                    const float sa = lds_sa[cur_stage * TM + wm * 64 + mt * 16 + frag_row];
-                    s0[mt] = sa * sw0;
-                    s1[mt] = sa * sw1;
-                }
-                i32x8 wf = wf_first;
-                f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
-#pragma unroll
-                for (int nt = 0; nt < 8; ++nt) {
-                    i32x8 wf_n = wf;
-                    if (nt + 1 < 8) wf_n = load_w(nt + 1);
-                    if (nt < 4 && more) issue_quarter(nt);
-                    const bool second = GMM1 ? (nt >= 4) : (wn == 1);
-#pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) {
-                        f32x4 nxt_part = part;
-                        if (mt < 3) nxt_part = mfma_fp8_16x16x128(wf, af[mt + 1]);
-                        else if (nt + 1 < 8) nxt_part = mfma_fp8_16x16x128(wf_n, af[0]);
-                        const float sc = second ? s1[mt] : s0[mt];
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
-                        part = nxt_part;
+                for (int mt = 0; mt < MT; ++mt) {
+                    const uint8_t *ab = sb + ((RG * mt + wm) * 16) * BKB;
+                    const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
+                    const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
+                    af[mt] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                    if (mt == 0 && MODE != MODE_W4A8) {
+                        /*
+                         * All waves start their fragment reads together after the barrier and the LDS serves them in the
+                         * order asked, so the two fragments of the first MFMA are asked for before the rest (measured,
+                         * alternating with the unordered build on one GPU: 1 % of the kernel; forcing the order of all of
+                         * them is slower).
+                         */
+                        wf_first = load_w(0);
+                        asm volatile("" ::: "memory");
                     }
-                    wf = wf_n;
                 }
-            } else if constexpr (MODE == MODE_W4A8) {
-                /*
-                 * The lane's 16 packed bytes are its 32 K values of this slab: dwords 0-1 unpack into the operand of the
-                 * first 64-deep MFMA, dwords 2-3 into the second (times 16: the nibble moves to the top of its byte,
-                 * which keeps the sign). The pair's int32 sum is promoted with the slab's group scales, and as in the
-                 * fp8 mode the MFMAs of pair p+1 are issued before the conversions and FMAs of pair p.
-                 */
-                const uint16_t *gsb = lds_gs + cur_stage * BN;
-                auto load_pk = [&](int nt) -> u32x4 { return *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + w4_off); };
-                auto load_gs = [&](int nt) -> u32x2 { return *reinterpret_cast<const u32x2 *>(gsb + lane_ch + w_ch[nt]); };
-                auto lo4 = [](uint32_t v) -> int { return (int)((v << 4) & 0xf0f0f0f0u); };
-                auto hi4 = [](uint32_t v) -> int { return (int)(v & 0xf0f0f0f0u); };
-                auto mfma_pair = [&](const u32x4 &pk, const i32x8 &a) -> i32x4 {
-                    const i32x4 w0 = i32x4{lo4(pk[0]), hi4(pk[0]), lo4(pk[1]), hi4(pk[1])};
-                    const i32x4 w1 = i32x4{lo4(pk[2]), hi4(pk[2]), lo4(pk[3]), hi4(pk[3])};
-                    i32x4 part = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, i32x4{a[0], a[1], a[2], a[3]}, i32x4{0, 0, 0, 0}, 0, 0, 0);
-                    return __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, i32x4{a[4], a[5], a[6], a[7]}, part, 0, 0, 0);
-                };
-                /* the packed chunk and the raw fp16 scales of the next channel sub-tile are fetched one sub-tile ahead */
-                u32x4 pk = load_pk(0);
-                u32x2 gsr = load_gs(0);
-                i32x4 part = mfma_pair(pk, af[0]);
+
+                if constexpr (MODE == MODE_FP8) {
+                    /*
+                     * Software pipeline over the 8 x MT (channel sub-tile, row sub-tile) pairs: the MFMA of pair p+1 is
+                     * issued before the four scale-and-accumulate FMAs of pair p, so the vector ALU works under the
+                     * matrix unit.
+                     */
+                    const float sw0 = sw_cur[kb], sw1 = sw_cur[D_MAX_KB + kb];
+                    float s0[MT], s1[MT];
 #pragma unroll
-                for (int nt = 0; nt < 8; ++nt) {
-                    u32x4 pkn = pk;
-                    u32x2 gsn = gsr;
-                    if (nt + 1 < 8) {
-                        pkn = load_pk(nt + 1);
-                        gsn = load_gs(nt + 1);
+                    for (int mt = 0; mt < MT; ++mt) {
+                        const float sa = lds_sa[cur_stage * TM + (RG * mt + wm) * 16 + frag_row];
+                        s0[mt] = sa * sw0;
+                        s1[mt] = sa * sw1;
                     }
-                    if (nt < 4 && more) issue_quarter(nt);
-                    const float gs[4] = {zb_fp16_to_f32(gsr[0] & 0xffffu), zb_fp16_to_f32(gsr[0] >> 16),
-                                         zb_fp16_to_f32(gsr[1] & 0xffffu), zb_fp16_to_f32(gsr[1] >> 16)};
+                    i32x8 wf = wf_first;
+                    f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
 #pragma unroll
-                    for (int mt = 0; mt < 4; ++mt) {
-                        i32x4 nxt_part = part;
-                        if (mt < 3) nxt_part = mfma_pair(pk, af[mt + 1]);
-                        else if (nt + 1 < 8) nxt_part = mfma_pair(pkn, af[0]);
+                    for (int nt = 0; nt < 8; ++nt) {
+                        i32x8 wf_n = wf;
+                        if (nt + 1 < 8) wf_n = load_w(nt + 1);
+                        if (nt < 4 && more) issue_quarter(nt);
+                        const bool second = GMM1 ? (nt >= 4) : (wn == 1);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf((float)part[i], gs[i], accf[mt][nt][i]);
-                        part = nxt_part;
+                        for (int mt = 0; mt < MT; ++mt) {
+                            f32x4 nxt_part = part;
+                            if (mt + 1 < MT) nxt_part = mfma_fp8_16x16x128(wf, af[mt + 1]);
+                            else if (nt + 1 < 8) nxt_part = mfma_fp8_16x16x128(wf_n, af[0]);
+                            const float sc = second ? s1[mt] : s0[mt];
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
+                            part = nxt_part;
+                        }
+                        wf = wf_n;
                     }
-                    pk = pkn;
-                    gsr = gsn;
-                }
-            } else {
-                /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
+                } else if constexpr (MODE == MODE_W4A8) {
+                    /*
+                     * The lane's 16 packed bytes are its 32 K values of this slab: dwords 0-1 unpack into the operand of
+                     * the first 64-deep MFMA, dwords 2-3 into the second (times 16: the nibble moves to the top of its
+                     * byte, which keeps the sign). The pair's int32 sum is promoted with the slab's group scales, and as
+                     * in the fp8 mode the MFMAs of pair p+1 are issued before the conversions and FMAs of pair p.
+                     */
+                    const uint16_t *gsb = lds_gs + cur_stage * BN;
+                    auto load_pk = [&](int nt) -> u32x4 { return *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + w4_off); };
+                    auto load_gs = [&](int nt) -> u32x2 { return *reinterpret_cast<const u32x2 *>(gsb + lane_ch + w_ch[nt]); };
+                    auto lo4 = [](uint32_t v) -> int { return (int)((v << 4) & 0xf0f0f0f0u); };
+                    auto hi4 = [](uint32_t v) -> int { return (int)(v & 0xf0f0f0f0u); };
+                    auto mfma_pair = [&](const u32x4 &pk, const i32x8 &a) -> i32x4 {
+                        const i32x4 w0 = i32x4{lo4(pk[0]), hi4(pk[0]), lo4(pk[1]), hi4(pk[1])};
+                        const i32x4 w1 = i32x4{lo4(pk[2]), hi4(pk[2]), lo4(pk[3]), hi4(pk[3])};
+                        i32x4 part = __builtin_amdgcn_mfma_i32_16x16x64_i8(w0, i32x4{a[0], a[1], a[2], a[3]}, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                        return __builtin_amdgcn_mfma_i32_16x16x64_i8(w1, i32x4{a[4], a[5], a[6], a[7]}, part, 0, 0, 0);
+                    };
+                    /* the packed chunk and the raw fp16 scales of the next channel sub-tile are fetched one sub-tile ahead */
+                    u32x4 pk = load_pk(0);
+                    u32x2 gsr = load_gs(0);
+                    i32x4 part = mfma_pair(pk, af[0]);
 #pragma unroll
-                for (int nt = 0; nt < 8; ++nt) {
-                    const i32x8 wf = nt == 0 ? wf_first : load_w(nt);
-                    if (nt < 4 && more) issue_quarter(nt);
-                    const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
+                    for (int nt = 0; nt < 8; ++nt) {
+                        u32x4 pkn = pk;
+                        u32x2 gsn = gsr;
+                        if (nt + 1 < 8) {
+                            pkn = load_pk(nt + 1);
+                            gsn = load_gs(nt + 1);
+                        }
+                        if (nt < 4 && more) issue_quarter(nt);
+                        const float gs[4] = {zb_fp16_to_f32(gsr[0] & 0xffffu), zb_fp16_to_f32(gsr[0] >> 16),
+                                             zb_fp16_to_f32(gsr[1] & 0xffffu), zb_fp16_to_f32(gsr[1] >> 16)};
 #pragma unroll
-                    for (int mt = 0; mt < 4; ++mt)
-                        if (!SKIP_ROW_GROUPS || mt < mt_act)
+                        for (int mt = 0; mt < MT; ++mt) {
+                            i32x4 nxt_part = part;
+                            if (mt + 1 < MT) nxt_part = mfma_pair(pk, af[mt + 1]);
+                            else if (nt + 1 < 8) nxt_part = mfma_pair(pkn, af[0]);
+#pragma unroll
+                            for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf((float)part[i], gs[i], accf[mt][nt][i]);
+                            part = nxt_part;
+                        }
+                        pk = pkn;
+                        gsr = gsn;
+                    }
+                } else {
+                    /* int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart */
+#pragma unroll
+                    for (int nt = 0; nt < 8; ++nt) {
+                        const i32x8 wf = nt == 0 ? wf_first : load_w(nt);
+                        if (nt < 4 && more) issue_quarter(nt);
+                        const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
                             acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
                                 wf0, i32x4{af[mt][0], af[mt][1], af[mt][2], af[mt][3]}, acci[mt][nt], 0, 0, 0);
 #pragma unroll
-                    for (int mt = 0; mt < 4; ++mt)
-                        if (!SKIP_ROW_GROUPS || mt < mt_act)
+                        for (int mt = 0; mt < MT; ++mt)
                             acci[mt][nt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(
                                 wf1, i32x4{af[mt][4], af[mt][5], af[mt][6], af[mt][7]}, acci[mt][nt], 0, 0, 0);
+                    }
                 }
             }
         }
+        };
+        if (mt_act == 4) k_loop(std::integral_constant<int, 4>{});
+        else if (mt_act == 3) k_loop(std::integral_constant<int, 3>{});
+        else if (mt_act == 2) k_loop(std::integral_constant<int, 2>{});
+        else if (mt_act == 1) k_loop(std::integral_constant<int, 1>{});
+        else k_loop(std::integral_constant<int, 0>{});
         if constexpr (MODE == MODE_W4A8) {      /* the unpacked weights were 16 x their value; a power of two divides out exactly */
 #pragma unroll
             for (int mt = 0; mt < 4; ++mt)
@@ -776,7 +792,7 @@ grouped_gemm_dma_kernel(GemmParams p)
         tc.expert = cur.expert;
         tc.m_tile = 0;
         tc.n_tile = cur.n_tile;
-        epilogue<MODE, GMM1, OUT_DT>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane, lds_rowmax, TM);
+        epilogue<MODE, GMM1, OUT_DT, RG>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane, lds_rowmax, TM);
         if (!nxt.valid) break;
         cur = nxt;
         sw_buf ^= 1;
