@@ -39,7 +39,7 @@ namespace {
 
 constexpr int BN = 256;          /* output channels per workgroup tile */
 constexpr int BKB = 128;         /* K bytes of an activation row per slab (128 int8/e4m3 elements) */
-constexpr int GROUP_N = 8;       /* channel tiles per schedule group */
+constexpr int GROUP_N = 8;       /* channel tiles per schedule group, at most */
 
 enum { MODE_W8A8 = 1, MODE_FP8 = 2, MODE_W4A8 = 3 };
 
@@ -279,7 +279,7 @@ struct DmaShape {
     static constexpr bool TWO_PHASE = TM == 256;            /* short tail tiles run after all the others (see the kernel) */
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 4 * D_MAX_KB * 4 +
                                      2 * (D_MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0) +
-                                     (TWO_PHASE ? D_MAX_EXPERTS * 2 : 0);
+                                     (TWO_PHASE ? D_MAX_EXPERTS * 2 + (D_MAX_EXPERTS + 1) * 4 : 0);
     static_assert(A_PARTS == 4 && PARTS % 4 == 0, "the issue schedule hands out a slab in four quarters");
     static_assert(NW <= HALF_BLOCKS && HALF_BLOCKS % NW == 0, "a wave's W blocks must not straddle a weight half");
     static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
@@ -358,7 +358,8 @@ grouped_gemm_dma_kernel(GemmParams p)
     int *lds_mtp = reinterpret_cast<int *>(lds_sw + 4 * D_MAX_KB);            /* [experts + 1] tiles of TM rows before expert e */
     int *lds_roff = lds_mtp + (D_MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
     uint16_t *lds_gs = reinterpret_cast<uint16_t *>(lds_roff + (D_MAX_EXPERTS + 1));   /* [NSTAGE][BN] W4A8 group scales (fp16) */
-    uint16_t *lds_tail = lds_gs + (WRB == 64 ? NSTAGE * BN : 0);                       /* [experts] experts with a short tail tile */
+    uint16_t *lds_tail = lds_gs + (WRB == 64 ? NSTAGE * BN : 0);                       /* [experts] the short experts, second phase */
+    int *lds_cost = reinterpret_cast<int *>(lds_tail + D_MAX_EXPERTS);                 /* [experts + 1] 16-row sub-tiles of the main tiles before expert e */
     constexpr bool TWO_PHASE = S::TWO_PHASE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -377,48 +378,55 @@ grouped_gemm_dma_kernel(GemmParams p)
      * also wait for the slabs in flight).
      */
     /*
-     * Tile order. A tail tile whose rows fill at most half of it keeps half of the waves idle and runs at the pace
-     * of its own loads; in the middle of the sequence it drifts away from the workgroups it shares slabs with, and
-     * the L2 stops serving them together (measured on 4096 tokens over 32 experts: 3.6 GB of HBM reads per launch
-     * for 1.25 GB of operands, against 1.45 GB when every expert has exactly 1024 rows). So such short tails (at most
-     * one per expert) are kept out of the main sequence and run after it, the longer class first: the tiles that
-     * run side by side take the same time. Same run time, 2.0 GB of HBM reads.
+     * Tile order. A tile with a few rows keeps most waves idle and runs at the pace of its own loads; in the middle
+     * of the sequence it drifts away from the workgroups it shares slabs with, and the L2 stops serving them
+     * together (measured on 4096 tokens over 32 experts with 42-row tail tiles in the sequence: 3.6 GB of HBM reads
+     * per launch for 1.25 GB of operands, against 1.45 GB when every expert has exactly 1024 rows). Rows are
+     * therefore cut into even tiles (fill_tile below), and the experts whose rows fill at most half a tile are kept
+     * out of the main sequence and run after it, the longer class first: tiles that run side by side take about the
+     * same time.
      */
     int n_tail = 0;
     if (wave == 0) {
-        int run = 0;
+        int run = 0, run_c = 0;
         for (int base = 0; base < E; base += 64) {
             const int e = base + lane;
-            int mt = 0;
+            int mt = 0, rows_e = 0;
             if (e < E) {
                 const int lo = p.row_off[e];
-                const int rows = p.row_off[e + 1] - lo;
-                mt = (rows + TM - 1) / TM;
-                if (TWO_PHASE && mt > 0 && rows - (mt - 1) * TM <= TM / 2) mt -= 1;      /* the short tail is not a main tile */
+                rows_e = p.row_off[e + 1] - lo;
+                mt = (rows_e + TM - 1) / TM;
+                if (TWO_PHASE && rows_e <= TM / 2) mt = 0;      /* a short expert's only tile is not a main tile */
                 lds_roff[e] = lo;
             }
-            int incl = mt;
+            /* what the expert's main tiles cost: their number times their height in 16-row sub-tiles (fill_tile cuts them evenly) */
+            const int cost = mt > 0 ? mt * ((((rows_e + mt - 1) / mt) + 15) >> 4) : 0;
+            int incl = mt, incl_c = cost;
 #pragma unroll
             for (int off = 1; off < 64; off <<= 1) {
-                const int o = __shfl_up(incl, off, 64);
-                if (lane >= off) incl += o;
+                const int o = __shfl_up(incl, off, 64), oc = __shfl_up(incl_c, off, 64);
+                if (lane >= off) { incl += o; incl_c += oc; }
             }
-            if (e < E) lds_mtp[e] = run + incl - mt;
+            if (e < E) {
+                lds_mtp[e] = run + incl - mt;
+                if (TWO_PHASE) lds_cost[e] = run_c + incl_c - cost;
+            }
             run += __shfl(incl, 63, 64);
+            run_c += __shfl(incl_c, 63, 64);
         }
         if (lane == 0) {
             lds_mtp[E] = run;
             lds_roff[E] = p.row_off[E];
+            if (TWO_PHASE) lds_cost[E] = run_c;
         }
         if (TWO_PHASE) {
-            for (int cls = 2; cls >= 1; --cls) {          /* tails of TM/4+1 .. TM/2 rows, then those of 1 .. TM/4 */
+            for (int cls = 2; cls >= 1; --cls) {          /* experts of TM/4+1 .. TM/2 rows, then those of 1 .. TM/4 */
                 for (int base = 0; base < E; base += 64) {
                     const int e = base + lane;
                     bool mine = false;
                     if (e < E) {
                         const int rows = p.row_off[e + 1] - p.row_off[e];
-                        const int tail = rows - (rows + TM - 1) / TM * TM + TM;          /* rows of the last tile, TM when it is full */
-                        mine = rows > 0 && tail <= TM / 2 && (tail > TM / 4) == (cls == 2);
+                        mine = rows > 0 && rows <= TM / 2 && (rows > TM / 4) == (cls == 2);
                     }
                     const uint64_t bal = __ballot(mine);
                     if (mine) lds_tail[n_tail + __popcll(bal & ((1ull << lane) - 1))] = (uint16_t)e;
@@ -433,17 +441,44 @@ grouped_gemm_dma_kernel(GemmParams p)
         n_tail = __builtin_amdgcn_readfirstlane(__float_as_int(lds_rowmax[0]));
         __syncthreads();
     }
-    /* XCD x (workgroups x, x+8, ...) owns the contiguous range [x*chunk, (x+1)*chunk) of the logical tile order */
+    /*
+     * XCD x (workgroups x, x+8, ...) owns a contiguous range of the logical tile order. Where tiles differ in height
+     * the ranges are cut at equal cost (16-row sub-tiles), not at equal tile counts: the kernel lasts as long as its
+     * slowest XCD.
+     */
     const int total = __builtin_amdgcn_readfirstlane(lds_mtp[E]) * n_tiles;
     const int chunk = (total + 7) / 8;
     const int xcd = blockIdx.x & 7, slots = gridDim.x >> 3;
-    const int lid_end = (xcd + 1) * chunk < total ? (xcd + 1) * chunk : total;
+    auto first_id_of = [&](int x) __attribute__((always_inline)) -> int {
+        if (!TWO_PHASE) return x * chunk < total ? x * chunk : total;
+        if (x >= 8) return total;
+        /* the tile at which the cost before it reaches x/8 of the whole: expert by search, tile within it by division */
+        const int64_t target = (int64_t)lds_cost[E] * n_tiles * x / 8;
+        int id = total;
+        for (int base = 0; base < E; base += 64) {
+            const int e = base + lane;
+            int64_t lo = INT64_MAX, hi = INT64_MAX;
+            if (e < E) { lo = (int64_t)lds_cost[e] * n_tiles; hi = (int64_t)lds_cost[e + 1] * n_tiles; }
+            const uint64_t bal = __ballot(lo <= target && target < hi);
+            if (bal) {
+                const int src = __ffsll((long long)bal) - 1;
+                const int ex = base + src;
+                const int mt_e = lds_mtp[ex + 1] - lds_mtp[ex];
+                const int height = (lds_cost[ex + 1] - lds_cost[ex]) / mt_e;      /* sub-tiles per tile of this expert */
+                id = lds_mtp[ex] * n_tiles + (int)((target - (int64_t)lds_cost[ex] * n_tiles) / height);
+                break;
+            }
+        }
+        return __builtin_amdgcn_readfirstlane(id);
+    };
+    const int lid_begin = first_id_of(xcd);
+    const int lid_end = first_id_of(xcd + 1);
     /* the short tails follow as ids total, total + 1, ...: n_tail * n_tiles of them, split over the XCDs the same way */
     const int total_b = n_tail * n_tiles;
     const int chunk_b = (total_b + 7) / 8;
     const int bid_begin = total + xcd * chunk_b + (blockIdx.x >> 3);
     const int bid_end = total + ((xcd + 1) * chunk_b < total_b ? (xcd + 1) * chunk_b : total_b);
-    int lid = xcd * chunk + (blockIdx.x >> 3);
+    int lid = lid_begin + (blockIdx.x >> 3);
     if (lid >= lid_end) lid = bid_begin;
     /* the id after `id` in this workgroup's sequence */
     auto next_id = [&](int id) __attribute__((always_inline)) {
@@ -454,9 +489,19 @@ grouped_gemm_dma_kernel(GemmParams p)
     auto fill_tile = [&](Tile &t, int expert, int n_tile, int m_tile) __attribute__((always_inline)) {
         t.expert = expert;
         t.n_tile = n_tile;
-        t.row_begin = __builtin_amdgcn_readfirstlane(lds_roff[expert]) + m_tile * TM;
-        t.row_end = __builtin_amdgcn_readfirstlane(lds_roff[expert + 1]);
-        t.last_rel = t.row_end - 1 - t.row_begin;   /* rows past the expert's end re-read its last row: in bounds, and one line */
+        /*
+         * An expert's rows are cut into its ceil(rows / TM) tiles evenly, in multiples of 16: 1066 rows are five tiles
+         * of 224, 224, 224, 224 and 170 rows rather than four of 256 and one of 42. The tiles cost what their 16-row
+         * sub-tiles cost (the K loop leaves out the absent ones), so this is no more work, and no tile is so short
+         * that it runs ahead of the tiles it shares slabs with.
+         */
+        const int first_row = __builtin_amdgcn_readfirstlane(lds_roff[expert]);
+        const int end_row = __builtin_amdgcn_readfirstlane(lds_roff[expert + 1]);
+        const int n_row_tiles = (end_row - first_row + TM - 1) / TM;
+        const int height = (((end_row - first_row + n_row_tiles - 1) / n_row_tiles) + 15) & ~15;
+        t.row_begin = first_row + m_tile * height;
+        t.row_end = t.row_begin + height < end_row ? t.row_begin + height : end_row;
+        t.last_rel = t.row_end - 1 - t.row_begin;   /* rows past the tile's end re-read its last row: in bounds, and one line */
         t.a_base = p.a + (int64_t)t.row_begin * K;
         t.sa_base = p.a_scale + (int64_t)t.row_begin * KB;
         /* weights come pre-packed as 16 KiB blocks of 128 channels x 128 K-bytes in LDS order ([E][N/128][K/128]) */
@@ -475,8 +520,7 @@ grouped_gemm_dma_kernel(GemmParams p)
         if (TWO_PHASE && id >= total) {              /* short tail number (id - total) / n_tiles, channel tile the remainder */
             const int j = (id - total) / n_tiles;
             const int expert = __builtin_amdgcn_readfirstlane((int)lds_tail[j]);
-            const int m_tile = __builtin_amdgcn_readfirstlane(lds_mtp[expert + 1] - lds_mtp[expert]);
-            fill_tile(t, expert, id - total - j * n_tiles, m_tile);
+            fill_tile(t, expert, id - total - j * n_tiles, 0);
             return;
         }
         const int q = id / n_tiles;                  /* index among all TM-row tiles: expert e has [mtp[e], mtp[e+1]) */
@@ -497,12 +541,17 @@ grouped_gemm_dma_kernel(GemmParams p)
         expert = __builtin_amdgcn_readfirstlane(expert);
         first = __builtin_amdgcn_readfirstlane(first);
         const int mt_e = __builtin_amdgcn_readfirstlane(next) - first;
-        /* within the expert: groups of GROUP_N channel tiles, row tiles fastest, so that concurrent tiles share slabs */
+        /*
+         * Within the expert: groups of (all its row tiles) x (a few channel tiles), row tile fastest, so that concurrent
+         * tiles share slabs: as many channel tiles as make the group fit the workgroups of one XCD, GROUP_N at most.
+         */
         const int l = id - first * n_tiles;
-        const int per_group = mt_e * GROUP_N;
+        int group_n = slots / mt_e;
+        group_n = group_n < 1 ? 1 : (group_n > GROUP_N ? GROUP_N : group_n);
+        const int per_group = mt_e * group_n;
         const int ng = l / per_group;
         const int r = l - ng * per_group;
-        fill_tile(t, expert, ng * GROUP_N + r / mt_e, r % mt_e);
+        fill_tile(t, expert, ng * group_n + r / mt_e, r % mt_e);
     };
 
     /*

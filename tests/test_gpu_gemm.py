@@ -131,6 +131,30 @@ def test_gemms_fp8_tile_order_with_short_tails(buf):
     y = gmm2(buf, dev(a), dev(sa), buf.prepack_weight(dev(w)), dev(sw), capi.DT_FP32, counts, K, N, 2)
     ref = zo.gmm2_fp8(a, sa, w, sw, counts)
     assert max_rel_err(zo.bf16_to_f32(host(y)), zo.bf16_to_f32(ref)) < 2e-2
+    q2, s2, _ = gmm1(buf, dev(a), dev(sa), buf.prepack_weight(dev(w)), dev(sw), counts, K, N, 2)
+    r_q2, r_s2, _ = zo.gmm1_swiglu_quant_fp8(a, sa, w, sw, counts)
+    got = zo.e4m3_to_f32(host(q2)).reshape(rows, N // 256, 128) * host(s2)[:, :, None]
+    want = zo.e4m3_to_f32(r_q2).reshape(rows, N // 256, 128) * r_s2[:, :, None]
+    assert np.allclose(host(s2), r_s2, rtol=1e-4)
+    assert_requant_close(got, want, host(q2), r_q2)
+
+
+def test_gemms_w8a8_even_row_tiles_in_the_few_row_shape_bit_exact(buf):
+    """At most 128 rows per expert on average selects the 128-row shape; the experts with more rows than that are cut
+    into even tiles there too (300 rows: 112 + 112 + 76), next to empty, one-row and exactly full experts."""
+    counts = np.array([300, 5, 0, 129, 128, 127, 17, 250, 1, 0, 33, 16], dtype=np.int64)
+    E, rows, K, N = len(counts), int(counts.sum()), 384, 512
+    assert rows <= 128 * E
+    a = rng(65).integers(-127, 128, (rows, K)).astype(np.int8)
+    xs = rng(66).uniform(0.005, 0.05, rows).astype(np.float32)
+    w = rng(67).integers(-16, 16, (E, K, N)).astype(np.int8)
+    ws = rng(68).uniform(0.0015, 0.0045, (E, N)).astype(np.float32)
+    y = gmm2(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), capi.DT_FP32, counts, K, N, 1)
+    assert np.array_equal(host(y), zo.grouped_gemm_w8a8_dequant(a, xs, w, ws, counts))
+    q2, s2, _ = gmm1(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), counts, K, N, 1)
+    r_q2, r_s2 = zo.gmm1_swiglu_quant_w8a8(a, xs, w, ws, counts)[:2]
+    assert np.array_equal(host(s2).view(np.uint32), r_s2.view(np.uint32))
+    assert np.array_equal(host(q2), r_q2)
 
 
 # ---- fp8 block-scaled ------------------------------------------------------------------------------------------
