@@ -157,6 +157,22 @@ def test_gemms_w8a8_even_row_tiles_in_the_few_row_shape_bit_exact(buf):
     assert np.array_equal(host(q2), r_q2)
 
 
+@pytest.mark.parametrize("rows", [40000, 200000])      # few rows per expert (128-row shape) / many (256-row shape)
+def test_gmm2_w8a8_largest_expert_count_bit_exact(buf, rows):
+    """1024 experts, the most the kernel's lookup tables hold: the tile lookup, the cost prefix and the list of short
+    experts all run over sixteen 64-expert chunks. Skewed counts leave many experts empty or short."""
+    E, K, N = 1024, 128, 256
+    g = rng(91)
+    counts = g.multinomial(rows, g.dirichlet(np.full(E, 0.3))).astype(np.int64)
+    assert (counts == 0).any() and counts.max() > 512
+    a = rng(92).integers(-127, 128, (rows, K)).astype(np.int8)
+    xs = rng(93).uniform(0.005, 0.05, rows).astype(np.float32)
+    w = rng(94).integers(-128, 128, (E, K, N)).astype(np.int8)
+    ws = rng(95).uniform(0.0015, 0.0045, (E, N)).astype(np.float32)
+    y = gmm2(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), capi.DT_FP32, counts, K, N, 1)
+    assert np.array_equal(host(y), zo.grouped_gemm_w8a8_dequant(a, xs, w, ws, counts))
+
+
 # ---- fp8 block-scaled ------------------------------------------------------------------------------------------
 
 def fp8_operands(E, K, N, rows, seed):
