@@ -276,7 +276,7 @@ struct DmaShape {
     static constexpr int A_PARTS = A_BYTES / 1024 / NW;    /* 1 KiB blocks of the A tile per wave (4) */
     static constexpr int W_PARTS = W_BYTES / 1024 / NW;    /* 1 KiB blocks of the W tile per wave (2, 4 or 8) */
     static constexpr int PARTS = W_PARTS > A_PARTS ? W_PARTS : A_PARTS;
-    static constexpr bool TWO_PHASE = TM == 256;            /* short tail tiles run after all the others (see the kernel) */
+    static constexpr bool TWO_PHASE = TM == 256;            /* the tiles of short experts run after all the others (see the kernel) */
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 4 * D_MAX_KB * 4 +
                                      2 * (D_MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0) +
                                      (TWO_PHASE ? D_MAX_EXPERTS * 2 + (D_MAX_EXPERTS + 1) * 4 : 0);
@@ -358,8 +358,8 @@ grouped_gemm_dma_kernel(GemmParams p)
     int *lds_mtp = reinterpret_cast<int *>(lds_sw + 4 * D_MAX_KB);            /* [experts + 1] tiles of TM rows before expert e */
     int *lds_roff = lds_mtp + (D_MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
     uint16_t *lds_gs = reinterpret_cast<uint16_t *>(lds_roff + (D_MAX_EXPERTS + 1));   /* [NSTAGE][BN] W4A8 group scales (fp16) */
-    uint16_t *lds_tail = lds_gs + (WRB == 64 ? NSTAGE * BN : 0);                       /* [experts] the short experts, second phase */
-    int *lds_cost = reinterpret_cast<int *>(lds_tail + D_MAX_EXPERTS);                 /* [experts + 1] 16-row sub-tiles of the main tiles before expert e */
+    uint16_t *lds_short = lds_gs + (WRB == 64 ? NSTAGE * BN : 0);                       /* [experts] the short experts, second phase */
+    int *lds_cost = reinterpret_cast<int *>(lds_short + D_MAX_EXPERTS);                 /* [experts + 1] 16-row sub-tiles of the main tiles before expert e */
     constexpr bool TWO_PHASE = S::TWO_PHASE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -386,7 +386,7 @@ grouped_gemm_dma_kernel(GemmParams p)
      * out of the main sequence and run after it, the longer class first: tiles that run side by side take about the
      * same time.
      */
-    int n_tail = 0;
+    int n_short = 0;
     if (wave == 0) {
         int run = 0, run_c = 0;
         for (int base = 0; base < E; base += 64) {
@@ -429,16 +429,16 @@ grouped_gemm_dma_kernel(GemmParams p)
                         mine = rows > 0 && rows <= TM / 2 && (rows > TM / 4) == (cls == 2);
                     }
                     const uint64_t bal = __ballot(mine);
-                    if (mine) lds_tail[n_tail + __popcll(bal & ((1ull << lane) - 1))] = (uint16_t)e;
-                    n_tail += __popcll(bal);
+                    if (mine) lds_short[n_short + __popcll(bal & ((1ull << lane) - 1))] = (uint16_t)e;
+                    n_short += __popcll(bal);
                 }
             }
-            if (lane == 0) lds_rowmax[0] = __int_as_float(n_tail);    /* for the other waves; the epilogues use this later */
+            if (lane == 0) lds_rowmax[0] = __int_as_float(n_short);    /* for the other waves; the epilogues use this later */
         }
     }
     __syncthreads();
     if (TWO_PHASE) {
-        n_tail = __builtin_amdgcn_readfirstlane(__float_as_int(lds_rowmax[0]));
+        n_short = __builtin_amdgcn_readfirstlane(__float_as_int(lds_rowmax[0]));
         __syncthreads();
     }
     /*
@@ -473,8 +473,8 @@ grouped_gemm_dma_kernel(GemmParams p)
     };
     const int lid_begin = first_id_of(xcd);
     const int lid_end = first_id_of(xcd + 1);
-    /* the short tails follow as ids total, total + 1, ...: n_tail * n_tiles of them, split over the XCDs the same way */
-    const int total_b = n_tail * n_tiles;
+    /* the short experts' tiles follow as ids total, total + 1, ...: n_short * n_tiles of them, split evenly over the XCDs */
+    const int total_b = n_short * n_tiles;
     const int chunk_b = (total_b + 7) / 8;
     const int bid_begin = total + xcd * chunk_b + (blockIdx.x >> 3);
     const int bid_end = total + ((xcd + 1) * chunk_b < total_b ? (xcd + 1) * chunk_b : total_b);
@@ -517,9 +517,9 @@ grouped_gemm_dma_kernel(GemmParams p)
     auto load_tile = [&](int id, Tile &t) __attribute__((always_inline)) {
         t.valid = id < total ? id < lid_end : id < bid_end;
         if (!t.valid) return;
-        if (TWO_PHASE && id >= total) {              /* short tail number (id - total) / n_tiles, channel tile the remainder */
+        if (TWO_PHASE && id >= total) {              /* short expert number (id - total) / n_tiles, channel tile the remainder */
             const int j = (id - total) / n_tiles;
-            const int expert = __builtin_amdgcn_readfirstlane((int)lds_tail[j]);
+            const int expert = __builtin_amdgcn_readfirstlane((int)lds_short[j]);
             fill_tile(t, expert, id - total - j * n_tiles, 0);
             return;
         }
