@@ -111,6 +111,34 @@ def test_dispatch_normal_bit_exact(buf, T, H, K, E, qmode):
         assert np.array_equal(host(scales)[:rows].view(np.uint32), r_scale.view(np.uint32))
 
 
+@pytest.mark.parametrize("T,H,K,E,qmode", [(4096, 7168, 8, 32, capi.QUANT_FP8_B128),      # the prefill share
+                                           (16384, 4096, 8, 128, capi.QUANT_INT8)])          # the W4A8 layer
+def test_dispatch_normal_full_size_bit_exact(buf, T, H, K, E, qmode):
+    x = bf16_normal((T, H), 31)
+    idx = distinct_topk(T, E, K, 32)
+    recv, scales, h, r_dest, r_scale, rows, put, r_send = run_dispatch(buf, x, zo.DT_BF16, idx, E, qmode)
+    assert rows == T * K
+    assert np.array_equal(host(recv)[:rows].view(r_dest.dtype), r_dest)
+    assert np.array_equal(host(scales)[:rows].view(np.uint32), r_scale.view(np.uint32))
+    # independent of the oracle: the rows are a permutation of the picks, expert-major and stable within an expert
+    dest_row = put[idx] + r_send
+    assert np.array_equal(np.sort(dest_row.ravel()), np.arange(rows))
+    order = np.argsort(dest_row.ravel(), kind="stable")
+    assert np.all(np.diff(idx.ravel()[order]) >= 0)
+    assert np.all(np.diff(order)[np.diff(idx.ravel()[order]) == 0] > 0)
+
+
+def test_combine_normal_full_size_round_trip(buf):
+    T, H, K, E = 4096, 7168, 8, 32
+    x = bf16_normal((T, H), 33)
+    idx = distinct_topk(T, E, K, 34)
+    w = rng(35).uniform(0.05, 1.0, (T, K)).astype(np.float32)
+    recv, _, h, r_dest, _, rows, put, r_send = run_dispatch(buf, x, zo.DT_BF16, idx, E, capi.NO_QUANT)
+    out = buf.combine(recv, h, dev(w))
+    assert np.array_equal(host(out), zo.combine(r_dest, zo.DT_BF16, put, w, idx.astype(np.int32), r_send, E))
+    assert calc_diff(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(x) * w.sum(1, keepdims=True)) < 5e-5
+
+
 def test_dispatch_fp16_input(buf):
     T, H, K, E = 40, 512, 4, 16
     x = zo.f32_to_fp16(rng(8).standard_normal((T, H)).astype(np.float32) * 3)
