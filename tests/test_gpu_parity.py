@@ -25,7 +25,8 @@ def buf():
 
 # ---- router ---------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("T,E,K", [(256, 8, 2), (300, 32, 8), (64, 128, 8), (17, 256, 6), (5, 1000, 32)])
+@pytest.mark.parametrize("T,E,K", [(256, 8, 2), (300, 32, 8), (64, 128, 8), (17, 256, 6), (5, 1000, 32), (4096, 32, 8),
+                                   (16384, 128, 8), (40, 65, 3), (9, 257, 4), (12, 64, 5)])
 def test_router(buf, T, E, K):
     logits = rng(T + E).standard_normal((T, E)).astype(np.float32)
     logits[0, :] = 0.5                       # all tied: lowest indices win
