@@ -346,6 +346,48 @@ def test_fused_moe_fp8(buf, T, H, K, E, I):
     assert calc_diff(f, r) < 1e-4
 
 
+@pytest.mark.parametrize("mode", [1, 2])
+def test_router_and_fused_moe_replay_from_a_hip_graph(buf, mode):
+    """The operator calls allocate nothing, wait for nothing and record no memset node, so the router and the fused
+    operator can be captured into a HIP graph. Every replay must give the eager result; the replays are separated by
+    the program's own eager launches and synchronisations."""
+    T, H, K, E, I = 96, 512, 4, 8, 256
+    _, _, _, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 90 + mode)
+    w1p, w2p = buf.prepack_weight(dev(w1)), buf.prepack_weight(dev(w2))
+    s1d, s2d = dev(s1), dev(s2, torch.bfloat16 if mode == 1 else None)
+    ws = torch.empty(buf.fused_workspace_bytes(T, H, K, E, 2 * I, mode), dtype=torch.uint8, device="cuda")
+    s_logits = torch.zeros((T, E), dtype=torch.float32, device="cuda")
+    s_x = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+    s_out = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+
+    def layer(logits, x, out, workspace):
+        idx, w = buf.topk_route(logits, K)
+        return buf.fused_deep_moe(x, idx, w1p, s1d, w2p, s2d, w, E, quant_mode=mode, workspace=workspace, out=out)
+
+    def inputs(seed):
+        lg = torch.from_numpy(rng(seed).standard_normal((T, E)).astype(np.float32)).cuda()
+        xx = torch.from_numpy(rng(seed + 1).uniform(-5, 5, (T, H)).astype(np.float32)).cuda().to(torch.bfloat16)
+        return lg, xx
+
+    layer(s_logits, s_x, s_out, ws)                      # first call outside the capture: one-time kernel attributes
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        _, _, g_nums = layer(s_logits, s_x, s_out, ws)
+    ws_eager = torch.empty_like(ws)
+    for seed in (200, 210, 220, 230):
+        lg, xx = inputs(seed)
+        e_out = torch.empty_like(s_out)
+        _, _, e_nums = layer(lg, xx, e_out, ws_eager)    # eager work between the replays
+        torch.cuda.synchronize()
+        s_logits.copy_(lg)
+        s_x.copy_(xx)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(g_nums, e_nums)
+        assert torch.equal(s_out.view(torch.int16), e_out.view(torch.int16)), "replay with seed %d differs from the eager call" % seed
+
+
 def test_prefill_share_full_size_sampled_tokens(buf):
     """The fp8 prefill share at its real size (4096 tokens x 7168, 32 experts, top-8, intermediate 2048). A token's
     output depends on its own row only (per-token quantisation, row-wise GEMMs, per-token combine), so the oracle is run
