@@ -48,6 +48,26 @@ ZBALHIP_API int32_t zbalhip_dispatch_layout(const void *topk_idx, int32_t idx_is
                                 int32_t *send_token_idx, int32_t *scratch, void *stream);
 
 /*
+ * zbalhip_dispatch_layout for callers that cannot allocate device memory
+ * (code under HIP graph capture, serving loops and harnesses that forbid
+ * hipMalloc). No counterpart in the reference. Same arguments, outputs and
+ * results as zbalhip_dispatch_layout, minus `scratch`: the per-block
+ * histograms live in a file-scope device array of the library
+ * (ZBALHIP_LAYOUT_MAX_BLOCKS * ZBALHIP_LAYOUT_STATIC_MAX_EXPERTS int32 =
+ * 200 KiB on every GPU the library runs on, held until the process ends).
+ * The call allocates and frees nothing. experts above
+ * ZBALHIP_LAYOUT_STATIC_MAX_EXPERTS is refused with -2 and a last-error text.
+ * All calls on one GPU share that array: calls that overlap on one GPU
+ * (different streams, different threads) race; order them on one stream.
+ * The first call on a GPU looks up the array's device address
+ * (hipGetSymbolAddress): make it before a graph capture starts.
+ */
+#define ZBALHIP_LAYOUT_STATIC_MAX_EXPERTS 1024
+ZBALHIP_API int32_t zbalhip_dispatch_layout_static(const void *topk_idx, int32_t idx_is_i64, int64_t tokens, int64_t experts,
+                                       int64_t topk, int32_t ranks, int32_t *tokens_per_rank,
+                                       int32_t *tokens_per_expert, int32_t *send_token_idx, void *stream);
+
+/*
  * Replaces ZBALOpNotifyDispatch (zbal_npu_operators.h:52-56; kernel
  * notify_dispatch.h:356-596) for one rank: recv_data [1,E] = counts,
  * put_offset [E] = exclusive cumsum, total_recv [1], recv_tokens_per_expert

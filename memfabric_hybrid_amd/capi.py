@@ -104,6 +104,7 @@ SIGNATURES = {
     # zbal_hip_kernels.h
     "zbalhip_topk_route": (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "zbalhip_dispatch_layout": (_i32, [_vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp]),
+    "zbalhip_dispatch_layout_static": (_i32, [_vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "zbalhip_dispatch_notify": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
     "zbalhip_dispatch_normal": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp]),
     "zbalhip_combine": (_i32, [_vp, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),

@@ -53,6 +53,9 @@ BootState &Boot()
 
 using namespace zbal;
 
+/* the kernel launchers' way to leave a last-error text (declared in kernels/zbal_device.h) */
+void zbalhip_set_last_error(const char *text) { ZBAL_LOG_AND_SET_LAST_ERROR(text); }
+
 extern "C" {
 
 __attribute__((visibility("default"))) const char *zbal_version() { return ZBAL_VERSION_STRING; }

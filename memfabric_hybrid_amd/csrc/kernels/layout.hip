@@ -12,6 +12,8 @@
  * by intersecting one ballot per index bit) and the four waves of a block
  * commit their running counts in wave order.
  */
+#include <mutex>
+
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
 
@@ -19,7 +21,31 @@
 #define ZB_LAYOUT_THREADS 256
 #define ZB_FUSED_THREADS 1024
 
+/*
+ * Per-block histograms of zbalhip_dispatch_layout_static: the rows its kernels otherwise find in the caller's
+ * `scratch` argument, for the largest case the entry point takes. Every GPU the library runs on holds its own copy
+ * for the life of the process (200 KiB). Host code never uses this name as an address: it asks the runtime for the
+ * device address once per device (static_scratch_of) and hands that pointer to the kernels.
+ */
+static __device__ __align__(256) int32_t scratch[ZBALHIP_LAYOUT_MAX_BLOCKS * ZB_MAX_EXPERTS];
+
 namespace {
+
+constexpr int ZB_MAX_DEVICES = 64;
+
+/* device address of this GPU's copy of `scratch`, looked up on the first call with that GPU current */
+int32_t *static_scratch_of(int dev)
+{
+    static std::mutex mu;
+    static int32_t *addr[ZB_MAX_DEVICES] = {};
+    std::lock_guard<std::mutex> guard(mu);
+    if (addr[dev] == nullptr) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return nullptr;
+        addr[dev] = static_cast<int32_t *>(p);
+    }
+    return addr[dev];
+}
 
 struct LayoutPlan {
     int nblk;
@@ -464,6 +490,30 @@ extern "C" int32_t zbalhip_dispatch_layout(const void *topk_idx, int32_t idx_is_
                                          (hipStream_t)stream);
     if (rc != ZBALHIP_OK) return rc;
     return zbalhip_scan_internal(scratch, nblk, experts, topk, 1, tokens_per_expert, nullptr, nullptr, nullptr, nullptr,
+                                 nullptr, nullptr, nullptr, (hipStream_t)stream);
+}
+
+extern "C" int32_t zbalhip_dispatch_layout_static(const void *topk_idx, int32_t idx_is_i64, int64_t tokens, int64_t experts,
+                                                  int64_t topk, int32_t ranks, int32_t *tokens_per_rank,
+                                                  int32_t *tokens_per_expert, int32_t *send_token_idx, void *stream)
+{
+    if (!topk_idx || !tokens_per_rank || !tokens_per_expert || !send_token_idx) return ZBALHIP_INVALID;
+    if (experts > ZBALHIP_LAYOUT_STATIC_MAX_EXPERTS) {
+        zbalhip_set_last_error("zbalhip_dispatch_layout_static: more experts than the static scratch holds (1024)");
+        return ZBALHIP_INVALID;
+    }
+    if (!layout_args_ok(tokens, experts, topk) || ranks <= 0 || ranks > experts || experts % ranks != 0)
+        return ZBALHIP_INVALID;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ZB_MAX_DEVICES) return ZBALHIP_RT_ERROR;
+    int32_t *hist = static_scratch_of(dev);
+    if (hist == nullptr) return ZBALHIP_RT_ERROR;
+    /* the histogram kernel writes every row that the rank and scan kernels read: nothing has to start at zero */
+    int nblk = 0;
+    int32_t rc = zbalhip_layout_internal(topk_idx, idx_is_i64, tokens, experts, topk, ranks, tokens_per_rank,
+                                         send_token_idx, hist, ZBALHIP_LAYOUT_MAX_BLOCKS, &nblk, (hipStream_t)stream);
+    if (rc != ZBALHIP_OK) return rc;
+    return zbalhip_scan_internal(hist, nblk, experts, topk, 1, tokens_per_expert, nullptr, nullptr, nullptr, nullptr,
                                  nullptr, nullptr, nullptr, (hipStream_t)stream);
 }
 

@@ -33,6 +33,9 @@ typedef int32_t i32x4 __attribute__((ext_vector_type(4)));
 typedef int32_t i32x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+/* thread-local last-error text of the library (zbal_get_last_error_msg), for launchers that refuse a call */
+void zbalhip_set_last_error(const char *text);
+
 static inline int32_t zbalhip_check_launch()
 {
     hipError_t e = hipGetLastError();
