@@ -9,10 +9,16 @@ GEMM 1 with SwiGLU + requantise, grouped GEMM 2, weighted combine), all through
 the zbal C ABI. The workload is the DeepSeek-V3-style prefill share: 4096
 tokens x hidden 7168, 32 local experts, top-8 over uniform-random logits, fp8
 e4m3 with 1x128 activation and 128x128 weight scales, intermediate 2048.
-Synthetic data, random weights. `--workload decode` (128 tokens, W8A8, Zipf(1.2)
-expert popularity), `--workload qwen_w4a8` (16384 tokens x hidden 4096, 128
-experts, W4A8) and `--workload reduce` measure the other configurations the same
-way; the default is the headline one.
+Synthetic data, random weights. The default run measures the headline workload
+and then, under `other_workloads` of the same JSON line, the other
+configurations the metric names: the 8 x 256 MiB local reduction (bf16 and
+fp32), the 128-token W8A8 decode layer with Zipf(1.2) expert popularity and the
+16384-token W4A8 layer. `--workload decode | qwen_w4a8 | reduce` measures one of
+them alone, with the full line.
+
+No cache flush between steps: one step streams 1.4 GB of weights and 0.9 GB of
+activations through a 32-MiB L2 and a 256-MiB memory-side cache, so every step
+starts cold (`config.l2_flush_between_steps` says so in the line).
 
 Prints ONE JSON line. `value` is tokens/s of the whole step. `roofline`
 prices the dominant kernel (grouped GEMM 1) from its algorithmic FLOPs and
@@ -52,6 +58,8 @@ def parse():
                     help="prefill = the headline fp8 MoE layer (default); decode = 128-token W8A8 layer with Zipf routing; "
                          "qwen_w4a8 = 16384-token W4A8 layer; reduce = the 8 x 256 MiB local reduction")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-others", action="store_true",
+                    help="headline workload only: leave out the `other_workloads` block (reduce, decode, W4A8)")
     return ap.parse_args()
 
 
@@ -73,12 +81,36 @@ def main():
     buf = Buffer()
     lib = buf.lib
     if args.workload == "reduce":
-        bench_reduce(args, torch, np, capi, buf)
-        buf.close()
-        return
-
-    bench_moe(args, torch, np, capi, buf, MOE_WORKLOADS[args.workload])
+        line = bench_reduce(args, torch, np, capi, buf)
+    else:
+        line = bench_moe(args, torch, np, capi, buf, args.workload)
+        if args.workload == "prefill" and not args.no_others and args.tokens == 4096:
+            # the rest of the metric (reduce % HBM, the decode and W4A8 layers), measured in the same run
+            line["other_workloads"] = other_workloads(args, torch, np, capi, buf)
+    print(json.dumps(line))
     buf.close()
+
+
+def other_workloads(args, torch, np, capi, buf):
+    """The configurations beside the headline one, each timed like it: `ms` per step, the dominant kernel's
+    algorithmic rate against its roofline, and whether the result matched the CPU oracle."""
+    out = []
+    red = bench_reduce(args, torch, np, capi, buf)
+    for name, v in red["variants"].items():
+        out.append({"workload": "local reduce-scatter shard, 8 x 256 MiB %s (BASELINE configs[3])" % name, "ms": v["ms"],
+                    "achieved": v["gbs"], "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": v["gbs"] / PEAK_HBM_GBS,
+                    "exact": v["exact"]})
+    torch.cuda.empty_cache()
+    for wl in ("decode", "qwen_w4a8"):
+        m = bench_moe(args, torch, np, capi, buf, wl)
+        r = m["roofline"]
+        out.append({"workload": m["config"]["workload"], "ms": m["ms_per_step"], "tokens_per_s": m["value"],
+                    "kernel": r["kernel"], "achieved": r["achieved"], "peak": r["peak"], "unit": r["unit"], "frac": r["frac"],
+                    "stages_ms": m["stages"]["ms"],
+                    "exact": None if m["parity"] is None else m["parity"]["bit_exact"],
+                    "parity_tokens": None if m["parity"] is None else m["parity"]["tokens"]})
+        torch.cuda.empty_cache()
+    return out
 
 
 # mode: zbal_fused_deep_moe quantMode (1 = W8A8, 2 = fp8 block-scaled, 3 = W4A8)
@@ -110,10 +142,11 @@ def make_weights(torch, buf, dev, mode, E, k, n):
     return w, buf.prepack_weight(w, int4=True), s
 
 
-def bench_moe(args, torch, np, capi, buf, cfg):
+def bench_moe(args, torch, np, capi, buf, workload):
+    cfg = MOE_WORKLOADS[workload]
     lib = buf.lib
     dev = torch.device("cuda", 0)
-    T = args.tokens if args.workload == "prefill" else cfg["T"]
+    T = args.tokens if workload == "prefill" else cfg["T"]
     H, E, K, I, mode = cfg["H"], cfg["E"], cfg["K"], cfg["I"], cfg["mode"]
     N1 = 2 * I
     rows = T * K
@@ -137,15 +170,14 @@ def bench_moe(args, torch, np, capi, buf, cfg):
 
     ws = torch.empty(buf.fused_workspace_bytes(T, H, K, E, N1, mode), dtype=torch.uint8, device=dev)
     out = torch.empty((T, H), dtype=torch.bfloat16, device=dev)
-    topk_idx = torch.empty((T, K), dtype=torch.int64, device=dev)
     topk_w = torch.empty((T, K), dtype=torch.float32, device=dev)
-    ids32 = torch.empty((T, K), dtype=torch.int32, device=dev)
+    ids32 = torch.empty((T, K), dtype=torch.int32, device=dev)   # the router writes the type the fused operator takes
     nums = torch.empty(E, dtype=torch.int64, device=dev)
 
     ti = capi.tensor_info
     null = capi.TensorInfo()
     wdt = {1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[mode]
-    d = dict(x=ti(x), logits=ti(logits), idx=ti(topk_idx), w=ti(topk_w), ids=ti(ids32),
+    d = dict(x=ti(x), logits=ti(logits), w=ti(topk_w), ids=ti(ids32),
              w1=ti(w1, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), s1=ti(s1),
              w2=ti(w2, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), s2=ti(s2),
              out=ti(out), nums=ti(nums), ws=ti(ws))
@@ -153,8 +185,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
     st = capi.stream_ptr()
 
     def step():
-        capi.check("route", lib.zbal_moe_topk_route(r(d["logits"]), K, r(d["idx"]), r(d["w"]), buf.comm, st, 0))
-        ids32.copy_(topk_idx)                            # the adaptor's int64 -> int32 cast (zbal_deepep.cpp:316)
+        capi.check("route", lib.zbal_moe_topk_route(r(d["logits"]), K, r(d["ids"]), r(d["w"]), buf.comm, st, 0))
         capi.check("fused", lib.zbal_fused_deep_moe(
             r(d["x"]), r(d["ids"]), r(d["w1"]), r(d["s1"]), r(d["w2"]), r(d["s2"]), r(d["w"]), r(null), r(null), r(null),
             r(null), r(null), r(null), r(null), r(d["out"]), r(null), r(d["nums"]), r(d["ws"]), E, mode, 0, N1, 0, 0,
@@ -183,8 +214,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
 
     def staged(evs):
         evs[0].record()
-        capi.check("route", lib.zbalhip_topk_route(logits.data_ptr(), T, E, K, topk_idx.data_ptr(), topk_w.data_ptr(), st))
-        ids32.copy_(topk_idx)
+        capi.check("route", lib.zbalhip_topk_route(logits.data_ptr(), T, E, K, ids32.data_ptr(), 0, topk_w.data_ptr(), st))
         evs[1].record()
         capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, None, T, H, K, E,
                                                               2 if mode == 2 else 1, q1, xs, eidx, nums.data_ptr(), row_off,
@@ -217,7 +247,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
     bytes_combine = rows * H * 2 + T * H * 2
     t1 = stage_ms["gmm1_swiglu_quant"] * 1e-3
     t2 = stage_ms["gmm2_dequant"] * 1e-3
-    if args.workload == "decode":
+    if workload == "decode":
         # a handful of rows per expert: the GEMMs stream the weights of the experts that received tokens
         touched = int((nums > 0).sum().item())
         wbytes1 = touched * H * N1
@@ -229,7 +259,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
         roofline = {"kernel": kname, "bound": "mfma", "achieved": flops1 / t1 / 1e12,
                     "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s" if mode == 2 else "TOP/s",
                     "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
-                    "traffic": GMM1_TRAFFIC_BYTES_T4096 if (args.workload == "prefill" and T == 4096) else None}
+                    "traffic": GMM1_TRAFFIC_BYTES_T4096 if (workload == "prefill" and T == 4096) else None}
     stages = {
         "ms": {k: round(v, 4) for k, v in stage_ms.items()},
         "gmm1_tflops": flops1 / t1 / 1e12,
@@ -245,7 +275,7 @@ def bench_moe(args, torch, np, capi, buf, cfg):
     parity = None
     if not args.no_cpu:
         from oracle import oracle as zo
-        ts = min(args.cpu_sample_tokens if args.workload == "prefill" else 128, T)
+        ts = min(args.cpu_sample_tokens if workload == "prefill" else 128, T)
 
         def h16(t):
             return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
@@ -274,10 +304,10 @@ def bench_moe(args, torch, np, capi, buf, cfg):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["name"], "tokens": T, "hidden": H, "experts": E, "topk": K, "intermediate": I,
-                   "quant": cfg["quant"], "parallelism": "1 GPU"},
+                   "quant": cfg["quant"], "parallelism": "1 GPU", "l2_flush_between_steps": False},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "parity": parity,
     }
-    print(json.dumps(line))
+    return line
 
 
 def bench_reduce(args, torch, np, capi, buf):
@@ -332,7 +362,7 @@ def bench_reduce(args, torch, np, capi, buf):
             "roofline": {"kernel": "reduce_kernel<bf16, sum, 8>", "bound": "hbm", "achieved": b["gbs"], "peak": PEAK_HBM_GBS,
                          "unit": "GB/s", "frac": b["gbs"] / PEAK_HBM_GBS, "traffic": REDUCE_TRAFFIC_BYTES},
             "cpu_baseline": None, "variants": results}
-    print(json.dumps(line))
+    return line
 
 
 def plan_workspace(lib, T, H, K, E, N1, qmode):

@@ -31,10 +31,12 @@ extern "C" {
 
 /*
  * Router (no reference counterpart). logits [T,E] fp32 -> topk_idx [T,K]
- * int64, topk_w [T,K] fp32. E <= 1024, K <= 32, K <= E.
+ * int64 (idx_is_i64 != 0, the type the layout operator takes) or int32 (the
+ * type the dispatch and fused operators take), topk_w [T,K] fp32.
+ * E <= 1024, K <= 32, K <= E.
  */
-ZBALHIP_API int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64_t experts, int64_t topk, int64_t *topk_idx,
-                           float *topk_w, void *stream);
+ZBALHIP_API int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64_t experts, int64_t topk, void *topk_idx,
+                           int32_t idx_is_i64, float *topk_w, void *stream);
 
 /*
  * Replaces ZBALOpDispatchLayout (zbal_npu_operators.h:47-50; kernel

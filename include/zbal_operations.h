@@ -154,7 +154,9 @@ uint64_t zbal_fused_deep_moe_workspace_size(int64_t tokens, int64_t hidden, int6
 
 /*
  * extension: softmax + top-k router. logits [T, E] fp32 -> topkIndex [T, K]
- * int64 and topkWeight [T, K] fp32 (probabilities renormalised over the K
+ * (int64, the type zbal_dispatch_normal_layout takes, or int32, the type
+ * the dispatch and fused operators take: the descriptor's dataType says
+ * which) and topkWeight [T, K] fp32 (probabilities renormalised over the K
  * picks). Picks are ordered by descending probability, ties to the lower
  * expert index. The reference has no router; its tests build these inputs
  * with torch.topk (test_low_latency.py:68-89).

@@ -130,9 +130,10 @@ class Buffer:
         return ctypes.byref(ti)
 
     # -- router (extension) ------------------------------------------------------------------
-    def topk_route(self, logits, num_topk):
+    def topk_route(self, logits, num_topk, idx_dtype=torch.int64):
+        """idx_dtype: torch.int64 (what get_dispatch_layout takes) or torch.int32 (what dispatch / fused_deep_moe take)"""
         T = logits.shape[0]
-        idx = self._empty((T, num_topk), torch.int64)
+        idx = self._empty((T, num_topk), idx_dtype)
         w = self._empty((T, num_topk), torch.float32)
         capi.check("zbal_moe_topk_route", self.lib.zbal_moe_topk_route(
             self._ti(logits), num_topk, self._ti(idx), self._ti(w), self.comm, capi.stream_ptr(), 0))

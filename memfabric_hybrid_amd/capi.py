@@ -102,7 +102,7 @@ SIGNATURES = {
     "zbal_moe_topk_route": (_i32, [_TI, _i64, _TI, _TI, _vp, _vp, _i64]),
     "zbal_moe_weight_prepack": (_i32, [_TI, _TI, _vp, _vp, _i64]),
     # zbal_hip_kernels.h
-    "zbalhip_topk_route": (_i32, [_vp, _i64, _i64, _i64, _vp, _vp, _vp]),
+    "zbalhip_topk_route": (_i32, [_vp, _i64, _i64, _i64, _vp, _i32, _vp, _vp]),
     "zbalhip_dispatch_layout": (_i32, [_vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp]),
     "zbalhip_dispatch_layout_static": (_i32, [_vp, _i32, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "zbalhip_dispatch_notify": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),

@@ -638,10 +638,12 @@ public:
                              op << " failed as experts " << E << " / topk " << topkNum << " are out of range", Z_INVALID_PARAM);
         if (T == 0) return Z_OK;
         ZB_CHECK(op, "logits", logits, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * E);
-        ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, T * topkNum);
+        /* int64 is what the layout operator takes, int32 what the dispatch and fused operators take */
+        ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT32, T * topkNum);
         ZB_CHECK(op, "topkWeight", topkWeight, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * topkNum);
-        return Launched(op, zbalhip_topk_route((const float *)logits->data, T, E, topkNum, (int64_t *)topkIndex->data,
-                                               (float *)topkWeight->data, stream));
+        return Launched(op, zbalhip_topk_route((const float *)logits->data, T, E, topkNum, topkIndex->data,
+                                               topkIndex->dataType == ZBAL_DATA_TYPE_INT64, (float *)topkWeight->data,
+                                               stream));
     }
 
     int32_t WeightPrepack(const zbal_tensor_info_t *src, const zbal_tensor_info_t *dst, aclrtStream stream, int64_t) override

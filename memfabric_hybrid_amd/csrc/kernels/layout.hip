@@ -321,8 +321,8 @@ layout_scan_kernel(const int32_t *__restrict__ hist, int nblk, int experts, int 
  */
 template <int PER_LANE>
 __global__ void __launch_bounds__(256)
-topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int topk, int64_t *__restrict__ topk_idx,
-                  float *__restrict__ topk_w)
+topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int topk, void *__restrict__ topk_idx,
+                  int idx_is_i64, float *__restrict__ topk_w)
 {
     const int lane = threadIdx.x & 63;
     const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
@@ -373,7 +373,8 @@ topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int
         if (lane == k) { myw = p; myidx = bidx; }
     }
     if (lane < topk) {
-        topk_idx[(int64_t)t * topk + lane] = myidx;
+        if (idx_is_i64) static_cast<int64_t *>(topk_idx)[(int64_t)t * topk + lane] = myidx;
+        else static_cast<int32_t *>(topk_idx)[(int64_t)t * topk + lane] = myidx;
         topk_w[(int64_t)t * topk + lane] = myw / wsum;
     }
 }
@@ -460,7 +461,7 @@ extern "C" int32_t zbalhip_fill_i32(int32_t *p, int64_t n, int32_t value, void *
 }
 
 extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64_t experts, int64_t topk,
-                                      int64_t *topk_idx, float *topk_w, void *stream)
+                                      void *topk_idx, int32_t idx_is_i64, float *topk_w, void *stream)
 {
     if (!logits || !topk_idx || !topk_w || tokens < 0 || experts <= 0 || experts > ZB_MAX_EXPERTS || topk <= 0 ||
         topk > 32 || topk > experts)
@@ -470,9 +471,9 @@ extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64
     const int64_t blocks = (tokens + wpb - 1) / wpb;
     const dim3 grid((unsigned)blocks), block(wpb * 64);
     hipStream_t st = (hipStream_t)stream;
-    if (experts <= 64) topk_route_kernel<1><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, topk_w);
-    else if (experts <= 256) topk_route_kernel<4><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, topk_w);
-    else topk_route_kernel<ZB_MAX_EXPERTS / 64><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, topk_w);
+    if (experts <= 64) topk_route_kernel<1><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
+    else if (experts <= 256) topk_route_kernel<4><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
+    else topk_route_kernel<ZB_MAX_EXPERTS / 64><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     return zbalhip_check_launch();
 }
 
