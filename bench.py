@@ -212,6 +212,8 @@ def bench_moe(args, torch, np, capi, buf, workload):
     names = ["route", "permute_quant", "gmm1_swiglu_quant", "gmm2_dequant", "combine"]
     s2dt = {1: capi.DT_BF16, 2: capi.DT_FP32, 3: capi.DT_FP16}[mode]
 
+    y_window = (ctypes.c_void_p * 1)(y)        # the one rank's window the expert outputs sit in
+
     def staged(evs):
         evs[0].record()
         capi.check("route", lib.zbalhip_topk_route(logits.data_ptr(), T, E, K, ids32.data_ptr(), 0, topk_w.data_ptr(), st))
@@ -226,8 +228,8 @@ def bench_moe(args, torch, np, capi, buf, workload):
         capi.check("gmm2", lib.zbalhip_gmm2_dequant(q2, sc2, w2.data_ptr(), s2.data_ptr(), s2dt, row_off, E, rows, I,
                                                     H, mode, capi.DT_BF16, y, st))
         evs[4].record()
-        capi.check("combine", lib.zbalhip_combine(y, capi.DT_BF16, row_off, 0, topk_w.data_ptr(), ids32.data_ptr(), eidx, T, H,
-                                                  K, E, out.data_ptr(), st))
+        capi.check("combine", lib.zbalhip_combine(y_window, 1, 0, rows, capi.DT_BF16, row_off, 0, topk_w.data_ptr(),
+                                                  ids32.data_ptr(), eidx, T, H, K, E, out.data_ptr(), st))
         evs[5].record()
 
     all_evs = [[torch.cuda.Event(enable_timing=True) for _ in range(6)] for _ in range(args.steps)]

@@ -10,9 +10,10 @@
  * Conventions: every pointer is a device pointer unless stated; `stream` is
  * a hipStream_t passed as void* (NULL = null stream); launches are
  * asynchronous; the return value is 0 or a negative ZResult (-2 invalid
- * parameter, -11 HIP runtime error). One rank (R = 1) owns all `experts`;
- * rows of the permuted activation matrix are expert-major in flat (t,k)
- * pick order. dtype arguments are zbal_datatype_t values.
+ * parameter, -11 HIP runtime error). Unless a function takes `ranks`, one
+ * rank owns all `experts`; rows of the permuted activation matrix are
+ * expert-major in flat (t,k) pick order. dtype arguments are zbal_datatype_t
+ * values.
  */
 #ifndef ZBAL_HIP_KERNELS_H_
 #define ZBAL_HIP_KERNELS_H_
@@ -71,35 +72,56 @@ ZBALHIP_API int32_t zbalhip_dispatch_layout_static(const void *topk_idx, int32_t
 
 /*
  * Replaces ZBALOpNotifyDispatch (zbal_npu_operators.h:52-56; kernel
- * notify_dispatch.h:356-596) for one rank: recv_data [1,E] = counts,
- * put_offset [E] = exclusive cumsum, total_recv [1], recv_tokens_per_expert
- * [E] i64, balance_matrix [1,2] = {0, tokens-1} (or {-1,-1} when no pick).
+ * notify_dispatch.h:356-596) from the point of view of rank `my_rank` of
+ * `ranks`. tokens_per_expert is a HOST array of `ranks` device pointers:
+ * entry s is rank s's per-expert counts [experts], read where they lie in that
+ * rank's window (one GPU: local allocations). Outputs: recv_data
+ * [ranks, experts] = the counts; put_offset [ranks * experts]: for every
+ * destination rank r, put_offset[r * experts + le * ranks + s] = exclusive
+ * running sum of counts[s][r * E_loc + le] in (local expert, source rank)
+ * order; total_recv [1] and recv_tokens_per_expert [experts / ranks] i64 for
+ * this rank; balance_matrix [ranks, 2 * ranks] = -1 except {0, tokens_i - 1}
+ * at [i, 2i], [i, 2i + 1] (no re-balancing). ranks == 1: put_offset is the
+ * exclusive cumsum of the counts and balance_matrix {0, tokens - 1}.
  */
-ZBALHIP_API int32_t zbalhip_dispatch_notify(const int32_t *tokens_per_expert, int64_t experts, int64_t topk, int32_t *recv_data,
-                                int32_t *put_offset, int32_t *total_recv, int64_t *recv_tokens_per_expert,
-                                int32_t *balance_matrix, void *stream);
+ZBALHIP_API int32_t zbalhip_dispatch_notify(const int32_t *const *tokens_per_expert, int32_t ranks, int32_t my_rank,
+                                int64_t experts, int64_t topk, int32_t *recv_data, int32_t *put_offset,
+                                int32_t *total_recv, int64_t *recv_tokens_per_expert, int32_t *balance_matrix,
+                                void *stream);
 
 /*
  * Replaces ZBALOpDispatchNormal (zbal_npu_operators.h:58-62; kernel
  * dispatch_normal.h:479-563). quant_mode: 0 copy, 1 int8 per token with
  * s = 127/(amax+1e-12), 2 e4m3 with 1x128 scales (dest_scale [rows, H/128]).
  * x_dtype: BFP16 or FP16. hidden % 16 == 0 (mode 2: % 128 == 0).
+ * dest / dest_scale are HOST arrays of `ranks` device pointers: the receive
+ * windows of the ranks (one GPU: local allocations; dest_scale may be null
+ * for mode 0). The row of a pick of global expert e goes to window
+ * e / (experts / ranks), row put_offset[e * ranks + my_rank] +
+ * send_token_idx (dispatch_normal.h:528-533). dest_rows = rows every window
+ * holds: a pick that would land past it is dropped, never written out of
+ * bounds.
  */
 ZBALHIP_API int32_t zbalhip_dispatch_normal(const void *x, int32_t x_dtype, const int32_t *topk_idx, const int32_t *send_token_idx,
                                 const int32_t *put_offset, int64_t tokens, int64_t hidden, int64_t topk,
-                                int64_t experts, int32_t quant_mode, void *dest, float *dest_scale, void *stream);
+                                int64_t experts, int32_t quant_mode, void *const *dest, float *const *dest_scale,
+                                int32_t ranks, int32_t my_rank, int64_t dest_rows, void *stream);
 
 /*
  * Replaces ZBALOpCombineNormal (zbal_npu_operators.h:64-68; kernel
- * combine_normal.h:398-494): out[t] = round(sum_k fp32(y[base[e]+idx]) * w),
- * multiply and add rounded separately, k ascending, invalid ids skipped; a
- * token with a valid id but send_token_idx < 0 is not written at all.
- * base_is_inclusive = 1 reads `base` as the low-latency kernels' inclusive
- * running counts (combine_low_latency.h:504-506).
+ * combine_normal.h:398-494): out[t] = round(sum_k fp32(row) * w), multiply
+ * and add rounded separately, k ascending, invalid ids skipped; a token with
+ * a valid id but send_token_idx < 0 is not written at all. y is a HOST array
+ * of `ranks` device pointers (the windows the rows were dispatched to, y_rows
+ * rows each; a row past that is skipped); the row of a pick of expert e is
+ * row base[e * ranks + my_rank] + send_token_idx of window e / (experts /
+ * ranks). base_is_inclusive = 1 (ranks == 1 only) reads `base` as the
+ * low-latency kernels' inclusive running counts (combine_low_latency.h:504-506).
  */
-ZBALHIP_API int32_t zbalhip_combine(const void *y, int32_t dtype, const int32_t *base, int32_t base_is_inclusive, const float *w,
-                        const int32_t *topk_idx, const int32_t *send_token_idx, int64_t tokens, int64_t hidden,
-                        int64_t topk, int64_t experts, void *out, void *stream);
+ZBALHIP_API int32_t zbalhip_combine(const void *const *y, int32_t ranks, int32_t my_rank, int64_t y_rows, int32_t dtype,
+                        const int32_t *base, int32_t base_is_inclusive, const float *w, const int32_t *topk_idx,
+                        const int32_t *send_token_idx, int64_t tokens, int64_t hidden, int64_t topk, int64_t experts,
+                        void *out, void *stream);
 
 /*
  * Replaces ZBALOpDispatchLowLatency (zbal_npu_operators.h:70-77; kernel

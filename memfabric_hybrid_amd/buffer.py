@@ -267,7 +267,8 @@ class Buffer:
     def fused_deep_moe(self, x, topk_idx, gmm1_permuted_weight, gmm1_permuted_weight_scale, gmm2_weight,
                        gmm2_weight_scale, topk_weights, num_experts, quant_mode=0, expert_smooth_scales=None,
                        share_gmm1_weight=None, share_gmm1_scale=None, share_gmm2_weight=None, share_gmm2_scale=None,
-                       share_smooth_scales=None, x_active_mask=None, workspace=None, out=None, is_tensor_list=False):
+                       share_smooth_scales=None, x_active_mask=None, workspace=None, out=None, is_tensor_list=False,
+                       share_out=None):
         """zbal_deepep.cpp:658-802. Weights are pre-packed (prepack_weight; shared-expert weights as [1,N,K]).
         Returns (output, share_output, expert_token_nums) like the reference; share_output is None without a shared
         expert. x_active_mask [T] bool: only the first sum(mask) tokens are routed; the other rows of `out` keep
@@ -283,7 +284,10 @@ class Buffer:
             workspace = self._empty((self.fused_workspace_bytes(T, H, K, num_experts, n1, quant_mode, sn1),), torch.uint8)
         if out is None:
             out = self._empty((T, H), x.dtype)
-        share_out = self._empty((T, H), x.dtype) if shared else None
+        if shared and share_out is None:
+            share_out = self._empty((T, H), x.dtype)
+        if not shared:
+            share_out = None
         token_nums = self._empty((num_experts,), torch.int64)
         wdt = {0: None, 1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[quant_mode]
         null = ctypes.byref(capi.TensorInfo())

@@ -24,7 +24,7 @@ PROBE = os.path.join(LIB_DIR, "gemm_ceiling_probe")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 KERNELS = ["layout", "dispatch", "combine", "reduce", "prepack", "gemm"]
-HOST = ["zbal_runtime", "zbal_registry", "zbal_gpu_communicator", "zbal_c_api"]
+HOST = ["zbal_runtime", "zbal_registry", "zbal_gpu_communicator", "zbal_c_api", "zbal_amd_operators"]
 
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-ffp-contract=off",

@@ -98,7 +98,7 @@ public:
     explicit GpuCommunicator(const GroupInfo &info) : Communicator(info)
     {
         const char *sw = std::getenv("ZBAL_PROF_ENABLE");
-        if (sw == nullptr || std::atoi(sw) != 1) return;
+        if (!info.traced || sw == nullptr || std::atoi(sw) != 1) return;
         int64_t points = 20480;
         if (const char *c = std::getenv("ZBAL_PROF_MAX_TRACING_COUNT")) {
             const long long v = std::atoll(c);
@@ -184,6 +184,12 @@ public:
     /* address of `p` (inside my window) in rank r's window */
     bool Translate(const char *op, const void *p, size_t bytes, const void **out) const
     {
+        if (info_.peerStride != 0) { /* symmetric address space: the same offset in every rank's slice */
+            const int64_t me = info_.worldRank[info_.myGroupRank];
+            for (uint16_t r = 0; r < info_.groupSize; ++r)
+                out[r] = static_cast<const uint8_t *>(p) + ((int64_t)info_.worldRank[r] - me) * (int64_t)info_.peerStride;
+            return true;
+        }
         const PeerWindow &mine = info_.peers[info_.myGroupRank];
         const uintptr_t a = reinterpret_cast<uintptr_t>(p), b = reinterpret_cast<uintptr_t>(mine.base);
         if (mine.base == nullptr || a < b || a + bytes > b + mine.size) {
@@ -199,6 +205,16 @@ public:
             out[r] = static_cast<const uint8_t *>(w.base) + (a - b);
         }
         return true;
+    }
+
+    /* the copies of `p` in every rank's window; a group of one needs no window: its only copy is `p` itself */
+    bool PeerCopies(const char *op, const void *p, size_t bytes, const void **out) const
+    {
+        if (info_.groupSize == 1 && info_.peerStride == 0 && info_.peers[0].base == nullptr) {
+            out[0] = p;
+            return true;
+        }
+        return Translate(op, p, bytes, out);
     }
 
     static size_t ElemSize(zbal_datatype_t dt)
@@ -229,7 +245,7 @@ public:
         }
         const size_t es = ElemSize(dt);
         const void *peer[ZBALHIP_MAX_REDUCE_PEERS];
-        if (info_.groupSize == 1 && info_.peers[0].base == nullptr) {
+        if (info_.groupSize == 1 && info_.peerStride == 0 && info_.peers[0].base == nullptr) {
             peer[0] = send; /* a group of one needs no window */
         } else if (!Translate(opName, send, (sliceOffsetElems + count) * es, peer)) {
             return Z_INVALID_PARAM;
@@ -286,16 +302,21 @@ public:
                                  aclrtStream stream, int64_t) override
     {
         const char *op = "NotifyDispatch";
-        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        const int64_t R = info_.groupSize, me = info_.myGroupRank;
         const int64_t E = sendCount; /* one count per expert, zbal_deepep.cpp:325-326 */
         ZBAL_VALIDATE_RETURN(E <= 1024, op << " failed as sendCount " << E << " exceeds 1024", Z_INVALID_PARAM);
+        ZBAL_VALIDATE_RETURN(R <= ZBALHIP_MAX_REDUCE_PEERS && E % R == 0,
+                             op << " failed as " << E << " experts do not split over a group of " << R, Z_INVALID_PARAM);
         ZB_CHECK(op, "sendTokensPerExpert", sendTokensPerExpert, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
-        ZB_CHECK(op, "recvBuff", recvBuff, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        ZB_CHECK(op, "recvBuff", recvBuff, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, R * E);
         ZB_CHECK(op, "totalRecvTokens", totalRecvTokens, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, 1);
-        ZB_CHECK(op, "recvTokensPerExpert", recvTokensPerExpert, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
-        ZB_CHECK(op, "pushTargetOffset", pushTargetOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
-        ZB_CHECK(op, "balanceMatrix", balanceMatrix, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, 2);
-        return Launched(op, zbalhip_dispatch_notify((const int32_t *)sendTokensPerExpert->data, E, topKNum,
+        ZB_CHECK(op, "recvTokensPerExpert", recvTokensPerExpert, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E / R);
+        ZB_CHECK(op, "pushTargetOffset", pushTargetOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, R * E);
+        ZB_CHECK(op, "balanceMatrix", balanceMatrix, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, R * 2 * R);
+        /* the counts of the other ranks are read where they lie: at the same offset in each rank's window */
+        const void *counts[ZBALHIP_MAX_REDUCE_PEERS];
+        if (!PeerCopies(op, sendTokensPerExpert->data, (size_t)E * 4, counts)) return Z_INVALID_PARAM;
+        return Launched(op, zbalhip_dispatch_notify((const int32_t *const *)counts, (int32_t)R, (int32_t)me, E, topKNum,
                                                     (int32_t *)recvBuff->data, (int32_t *)pushTargetOffset->data,
                                                     (int32_t *)totalRecvTokens->data,
                                                     (int64_t *)recvTokensPerExpert->data,
@@ -320,7 +341,9 @@ public:
                            aclrtStream stream, int64_t) override
     {
         const char *op = "DispatchNormal";
-        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        const int64_t R = info_.groupSize, me = info_.myGroupRank;
+        ZBAL_VALIDATE_RETURN(R <= ZBALHIP_MAX_REDUCE_PEERS && expertNum % R == 0,
+                             op << " failed as " << expertNum << " experts do not split over a group of " << R, Z_INVALID_PARAM);
         int64_t T = 0, H = 0;
         if (!TokensShape(op, srcTokens, &T, &H)) return Z_INVALID_PARAM;
         ZBAL_VALIDATE_RETURN(topkIndex->dim == 2 && topkIndex->shape[0] == T, op << " failed as topkIndex must be [tokens, topk]",
@@ -337,21 +360,35 @@ public:
         ZB_CHECK(op, "srcTokens", srcTokens, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
         ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
         ZB_CHECK(op, "sendTokensIndex", sendTokensIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
-        ZB_CHECK(op, "pushTargetOffset", pushTargetOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum);
+        ZB_CHECK(op, "pushTargetOffset", pushTargetOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum * R);
+        int64_t scalesPerRow = 0;
         if (quantMode == NO_QUANT) {
             ZB_CHECK(op, "destTokens", destTokens, srcTokens->dataType, srcTokens->dataType, H);
         } else if (quantMode == QUANT_BF16_2_INT8) {
             ZB_CHECK(op, "destTokens", destTokens, ZBAL_DATA_TYPE_INT8, ZBAL_DATA_TYPE_INT8, H);
             ZB_CHECK(op, "destScale", destScale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, 1);
+            scalesPerRow = 1;
         } else {
             ZB_CHECK(op, "destTokens", destTokens, ZBAL_DATA_TYPE_FP8_E4M3, ZBAL_DATA_TYPE_UINT8, H);
             ZB_CHECK(op, "destScale", destScale, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, H / 128);
+            scalesPerRow = H / 128;
         }
+        /*
+         * The receive tensors may be sized from the received-token total (the reference does, zbal_deepep.cpp:359-375):
+         * the kernel gets the number of rows they hold and drops what would land past it instead of writing there.
+         */
+        int64_t destRows = Numel(destTokens) / H;
+        if (scalesPerRow > 0 && Numel(destScale) / scalesPerRow < destRows) destRows = Numel(destScale) / scalesPerRow;
+        /* rank r's receive tensors sit at the same offset in rank r's window */
+        const void *dest[ZBALHIP_MAX_REDUCE_PEERS], *scale[ZBALHIP_MAX_REDUCE_PEERS] = {};
+        if (!PeerCopies(op, destTokens->data, (size_t)destRows * rowBytes, dest)) return Z_INVALID_PARAM;
+        if (scalesPerRow > 0 && !PeerCopies(op, destScale->data, (size_t)destRows * scalesPerRow * 4, scale)) return Z_INVALID_PARAM;
         return Launched(op, zbalhip_dispatch_normal(srcTokens->data, srcTokens->dataType, (const int32_t *)topkIndex->data,
                                                     (const int32_t *)sendTokensIndex->data,
                                                     (const int32_t *)pushTargetOffset->data, T, H, K, expertNum,
-                                                    (int32_t)quantMode, destTokens->data, (float *)destScale->data,
-                                                    stream));
+                                                    (int32_t)quantMode, (void *const *)dest,
+                                                    scalesPerRow > 0 ? (float *const *)scale : nullptr, (int32_t)R,
+                                                    (int32_t)me, destRows, stream));
     }
 
     int32_t CombineNormal(const zbal_tensor_info_t *srcTokens, const zbal_tensor_info_t *srcTokensPerEp,
@@ -360,7 +397,9 @@ public:
                           const zbal_tensor_info_t *destTokens, aclrtStream stream, int64_t) override
     {
         const char *op = "CombineNormal";
-        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        const int64_t R = info_.groupSize, me = info_.myGroupRank;
+        ZBAL_VALIDATE_RETURN(R <= ZBALHIP_MAX_REDUCE_PEERS && expertNum % R == 0,
+                             op << " failed as " << expertNum << " experts do not split over a group of " << R, Z_INVALID_PARAM);
         int64_t T = 0, H = 0;
         if (!TokensShape(op, destTokens, &T, &H)) return Z_INVALID_PARAM;
         ZBAL_VALIDATE_RETURN(topkIndex->dim == 2 && topkIndex->shape[0] == T, op << " failed as topkIndex must be [tokens, topk]",
@@ -374,14 +413,18 @@ public:
         ZBAL_VALIDATE_RETURN(srcTokens->dataType == destTokens->dataType, op << " failed as source and destination types differ",
                              Z_INVALID_PARAM);
         ZB_CHECK(op, "destTokens", destTokens, srcTokens->dataType, srcTokens->dataType, T * H);
-        ZB_CHECK(op, "srcTokensPerEp", srcTokensPerEp, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum);
+        ZB_CHECK(op, "srcTokensPerEp", srcTokensPerEp, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, expertNum * R);
         ZB_CHECK(op, "topKWeight", topKWeight, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
         ZB_CHECK(op, "topkIndex", topkIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
         ZB_CHECK(op, "sendTokensIndex", sendTokensIndex, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
-        return Launched(op, zbalhip_combine(srcTokens->data, srcTokens->dataType, (const int32_t *)srcTokensPerEp->data, 0,
-                                            (const float *)topKWeight->data, (const int32_t *)topkIndex->data,
-                                            (const int32_t *)sendTokensIndex->data, T, H, K, expertNum,
-                                            destTokens->data, stream));
+        /* the expert outputs are read from the window of the rank that owns the expert; rows past what they hold are skipped */
+        const int64_t srcRows = Numel(srcTokens) / H;
+        const void *src[ZBALHIP_MAX_REDUCE_PEERS];
+        if (!PeerCopies(op, srcTokens->data, (size_t)srcRows * H * 2, src)) return Z_INVALID_PARAM;
+        return Launched(op, zbalhip_combine(src, (int32_t)R, (int32_t)me, srcRows, srcTokens->dataType,
+                                            (const int32_t *)srcTokensPerEp->data, 0, (const float *)topKWeight->data,
+                                            (const int32_t *)topkIndex->data, (const int32_t *)sendTokensIndex->data, T, H, K,
+                                            expertNum, destTokens->data, stream));
     }
 
     int32_t DispatchLowLatency(const zbal_tensor_info_t *x, const zbal_tensor_info_t *expertIds, int64_t moeExpertNum,
@@ -412,17 +455,20 @@ public:
         ZB_CHECK(op, "expertTokenNumsOut", expertTokenNumsOut, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
         ZB_CHECK(op, "epRecvCountsOut", epRecvCountsOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
         ZB_CHECK(op, "putOffset", putOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
-        ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
-        ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
-        ZB_CHECK(op, "expandIdxOut", expandIdxOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
-        /* every pick may be valid, so the packed output must hold tokens * topk rows */
-        if (quantMode == 0) {
-            ZB_CHECK(op, "expandXOut", expandXOut, x->dataType, x->dataType, T * K * H);
-        } else {
-            ZB_CHECK(op, "expandXOut", expandXOut, quantMode == 1 ? ZBAL_DATA_TYPE_INT8 : ZBAL_DATA_TYPE_FP8_E4M3,
-                     quantMode == 1 ? ZBAL_DATA_TYPE_INT8 : ZBAL_DATA_TYPE_UINT8, T * K * H);
-            ZB_CHECK(op, "dynamicScalesOut", dynamicScalesOut, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32,
-                     quantMode == 1 ? T * K : T * K * (H / 128));
+        /* an empty batch has empty per-token tensors (torch hands out a null pointer for them): only the counts are written */
+        if (T > 0) {
+            ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
+            ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+            ZB_CHECK(op, "expandIdxOut", expandIdxOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+            /* every pick may be valid, so the packed output must hold tokens * topk rows */
+            if (quantMode == 0) {
+                ZB_CHECK(op, "expandXOut", expandXOut, x->dataType, x->dataType, T * K * H);
+            } else {
+                ZB_CHECK(op, "expandXOut", expandXOut, quantMode == 1 ? ZBAL_DATA_TYPE_INT8 : ZBAL_DATA_TYPE_FP8_E4M3,
+                         quantMode == 1 ? ZBAL_DATA_TYPE_INT8 : ZBAL_DATA_TYPE_UINT8, T * K * H);
+                ZB_CHECK(op, "dynamicScalesOut", dynamicScalesOut, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32,
+                         quantMode == 1 ? T * K : T * K * (H / 128));
+            }
         }
         int64_t blocks = Numel(putOffset) / E;
         if (blocks > ZBALHIP_LAYOUT_MAX_BLOCKS) blocks = ZBALHIP_LAYOUT_MAX_BLOCKS;
@@ -459,10 +505,11 @@ public:
         ZB_CHECK(op, "expertIdx", expertIdx, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
         ZB_CHECK(op, "epSendCounts", epSendCounts, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, moeExpertNum);
         ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
-        return Launched(op, zbalhip_combine(expandX->data, expandX->dataType, (const int32_t *)epSendCounts->data, 1,
-                                            (const float *)expertScales->data, (const int32_t *)expertIds->data,
-                                            (const int32_t *)expertIdx->data, T, H, K, moeExpertNum, xOut->data,
-                                            stream));
+        const void *src[1] = {expandX->data};
+        return Launched(op, zbalhip_combine(src, 1, 0, Numel(expandX) / H, expandX->dataType,
+                                            (const int32_t *)epSendCounts->data, 1, (const float *)expertScales->data,
+                                            (const int32_t *)expertIds->data, (const int32_t *)expertIdx->data, T, H, K,
+                                            moeExpertNum, xOut->data, stream));
     }
 
     /* shapes and types of one FFN's weights and scales: `experts` experts of [H, N1] and [N1/2, H] */
@@ -531,10 +578,15 @@ public:
         ZBAL_VALIDATE_RETURN(K <= 32, op << " failed as topk " << K << " exceeds 32", Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(E <= 1024, op << " failed as moeExpertNum exceeds 1024", Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(H % 256 == 0, op << " failed as hidden " << H << " must be a multiple of 256", Z_INVALID_PARAM);
-        ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
-        ZB_CHECK(op, "output", output, x->dataType, x->dataType, T * H);
-        ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
-        ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
+        if (T > 0) { /* an empty batch has empty per-token tensors (null data): only expertTokenNums is written */
+            ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
+            ZB_CHECK(op, "output", output, x->dataType, x->dataType, T * H);
+            ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
+            ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
+        } else {
+            ZBAL_VALIDATE_RETURN(x->dataType == ZBAL_DATA_TYPE_BFP16 || x->dataType == ZBAL_DATA_TYPE_FP16,
+                                 op << " failed as x has type " << DtName(x->dataType), Z_INVALID_PARAM);
+        }
         ZB_CHECK(op, "expertTokenNums", expertTokenNums, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
         int wscale2Dt = ZBAL_DATA_TYPE_FP32, shareWscale2Dt = ZBAL_DATA_TYPE_FP32;
         if (!CheckFfnWeights(op, "expert", mode, E, H, N1, gmm1Weight, gmm1Scale, gmm2Weight, gmm2Scale, &wscale2Dt))
@@ -549,7 +601,7 @@ public:
             if (!CheckFfnWeights(op, "shared", mode, 1, H, SN1, shareGmm1Weight, shareGmm1Scale, shareGmm2Weight,
                                  shareGmm2Scale, &shareWscale2Dt))
                 return Z_INVALID_PARAM;
-            ZB_CHECK(op, "shareOutput", shareOutput, x->dataType, x->dataType, T * H);
+            if (T > 0) ZB_CHECK(op, "shareOutput", shareOutput, x->dataType, x->dataType, T * H);
             if (shareSmoothScales && shareSmoothScales->data) {
                 ZBAL_VALIDATE_RETURN(mode != 2, op << " failed as smooth scales do not apply to the fp8 mode", Z_INVALID_PARAM);
                 ZB_CHECK(op, "shareSmoothScales", shareSmoothScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, H);
@@ -558,7 +610,7 @@ public:
         }
         const uint8_t *activeMask = nullptr;
         if (xActiveMask && xActiveMask->data) { /* one bool per token; the first sum(mask) tokens are routed */
-            ZB_CHECK(op, "xActiveMask", xActiveMask, ZBAL_DATA_TYPE_UINT8, ZBAL_DATA_TYPE_INT8, T);
+            if (T > 0) ZB_CHECK(op, "xActiveMask", xActiveMask, ZBAL_DATA_TYPE_UINT8, ZBAL_DATA_TYPE_INT8, T);
             activeMask = (const uint8_t *)xActiveMask->data;
         }
         FusedWorkspace ws;
@@ -603,7 +655,8 @@ public:
             int64_t *shareCount = (int64_t *)((uint8_t *)y + Align256((uint64_t)T * 4));
             rc = zbalhip_fill_i32(zeroIds, T, 0, stream);
             if (rc != 0) return Launched(op, rc);
-            rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, nullptr, T, H, 1, 1, qmode, q1, xs, expandIdx,
+            /* with x_active_mask the shared expert, too, sees only the first sum(mask) tokens (TokenActiveMaskCal) */
+            rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, activeMask, T, H, 1, 1, qmode, q1, xs, expandIdx,
                                              shareCount, rowOff, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
             if (rc != 0) return Launched(op, rc);
             rc = zbalhip_gmm1_swiglu_quant(q1, xs, shareGmm1Weight->data, shareGmm1Scale->data, rowOff, 1, T, H, SN1, mode,
@@ -623,7 +676,8 @@ public:
         rc = zbalhip_gmm2_dequant(q2, scale2, gmm2Weight->data, gmm2Scale->data, wscale2Dt, rowOff, E, rows, I, H, gemmMode,
                                   x->dataType, y, stream);
         if (rc != 0) return Launched(op, rc);
-        return Launched(op, zbalhip_combine(y, x->dataType, rowOff, 0, (const float *)expertScales->data,
+        const void *ySrc[1] = {y};
+        return Launched(op, zbalhip_combine(ySrc, 1, 0, rows, x->dataType, rowOff, 0, (const float *)expertScales->data,
                                             (const int32_t *)expertIds->data, expandIdx, T, H, K, E, output->data,
                                             stream));
     }

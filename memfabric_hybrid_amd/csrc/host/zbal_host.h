@@ -108,6 +108,14 @@ struct GroupInfo {
     uint32_t groupIndex = 0;
     zbal_backend_t backend = ZBAL_AMD_GPU;
     std::vector<PeerWindow> peers; /* one per group rank */
+    /*
+     * The reference's symmetric address space instead of registered windows: group rank r's copy of a tensor lies
+     * (worldRank[r] - worldRank[me]) * peerStride bytes from this rank's (CommGroupInfo::localDeviceMemSize and
+     * peerGroupRank2WorldRank). Used when peerStride != 0; the launchers of zbal_amd_operators.h fill it in.
+     */
+    uint64_t peerStride = 0;
+    std::vector<uint16_t> worldRank;
+    bool traced = true;            /* false: never owns a trace ring, whatever ZBAL_PROF_ENABLE says */
 };
 
 class Communicator {

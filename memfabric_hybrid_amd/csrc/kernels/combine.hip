@@ -17,14 +17,25 @@ constexpr int kThreads = 256;
 constexpr int kMaxTopk = 32;
 constexpr int kGroup = 8;
 
+/*
+ * Where the rows are read from: expert e's rows sit in the window of rank e / e_loc, at the slot
+ * base[e * ranks + my_rank] that this rank's dispatch wrote them to (reference zbal_kernel_combine_normal.h:437-494).
+ * One GPU: the windows are local allocations; over xGMI they would be mapped peer memory. rows_cap: rows per window.
+ */
+struct PeerSource {
+    const uint16_t *y[ZBALHIP_MAX_REDUCE_PEERS];
+    int ranks, my_rank, e_loc;
+    int64_t rows_cap;
+};
+
 template <int DT>
 __global__ void __launch_bounds__(kThreads)
-combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base, int base_inclusive,
+combine_kernel(PeerSource src, const int32_t *__restrict__ base, int base_inclusive,
                const float *__restrict__ w, const int32_t *__restrict__ topk_idx,
                const int32_t *__restrict__ rank_in_expert, int hidden, int topk, int experts,
                uint16_t *__restrict__ out)
 {
-    __shared__ int64_t s_row[kMaxTopk];
+    __shared__ const uint16_t *s_row[kMaxTopk];
     __shared__ float s_w[kMaxTopk];
     __shared__ int s_n;
     const int t = blockIdx.x;
@@ -39,8 +50,11 @@ combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base,
             if (e < 0 || e >= experts) continue;
             const int32_t rk = rank_in_expert[(int64_t)t * topk + k];
             if (rk < 0) { n = -1; break; }
-            const int32_t b = base_inclusive ? (e == 0 ? 0 : base[e - 1]) : base[e];
-            s_row[n] = (int64_t)b + rk;
+            const int slot = e * src.ranks + src.my_rank;
+            const int32_t b = base_inclusive ? (slot == 0 ? 0 : base[slot - 1]) : base[slot];
+            const int64_t row = (int64_t)b + rk;
+            if (row >= src.rows_cap) continue;            /* never read past the window */
+            s_row[n] = src.y[e / src.e_loc] + row * hidden;
             s_w[n] = w[(int64_t)t * topk + k];
             ++n;
         }
@@ -60,7 +74,7 @@ combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base,
             for (int u = 0; u < kGroup; ++u)
                 if (k0 + u < n)
                     v[u] = __builtin_nontemporal_load(
-                        reinterpret_cast<const u32x4 *>(y + s_row[k0 + u] * hidden + (int64_t)c * 8));
+                        reinterpret_cast<const u32x4 *>(s_row[k0 + u] + (int64_t)c * 8));
 #pragma unroll
             for (int u = 0; u < kGroup; ++u) {
                 if (k0 + u < n) {
@@ -84,26 +98,36 @@ combine_kernel(const uint16_t *__restrict__ y, const int32_t *__restrict__ base,
 
 } // namespace
 
-extern "C" int32_t zbalhip_combine(const void *y, int32_t dtype, const int32_t *base, int32_t base_is_inclusive,
-                                   const float *w, const int32_t *topk_idx, const int32_t *send_token_idx,
-                                   int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, void *out,
-                                   void *stream)
+extern "C" int32_t zbalhip_combine(const void *const *y, int32_t ranks, int32_t my_rank, int64_t y_rows, int32_t dtype,
+                                   const int32_t *base, int32_t base_is_inclusive, const float *w, const int32_t *topk_idx,
+                                   const int32_t *send_token_idx, int64_t tokens, int64_t hidden, int64_t topk,
+                                   int64_t experts, void *out, void *stream)
 {
     if (!y || !base || !w || !topk_idx || !send_token_idx || !out) return ZBALHIP_INVALID;
     if (dtype != ZDT_BF16 && dtype != ZDT_FP16) return ZBALHIP_INVALID;
     if (tokens < 0 || hidden <= 0 || hidden % 8 != 0 || topk <= 0 || topk > kMaxTopk || experts <= 0)
         return ZBALHIP_INVALID;
+    if (ranks <= 0 || ranks > ZBALHIP_MAX_REDUCE_PEERS || my_rank < 0 || my_rank >= ranks || experts % ranks != 0 || y_rows < 0)
+        return ZBALHIP_INVALID;
+    if (base_is_inclusive && ranks != 1) return ZBALHIP_INVALID;
+    PeerSource src = {};
+    for (int r = 0; r < ranks; ++r) {
+        if (!y[r]) return ZBALHIP_INVALID;
+        src.y[r] = (const uint16_t *)y[r];
+    }
+    src.ranks = ranks;
+    src.my_rank = my_rank;
+    src.e_loc = (int)(experts / ranks);
+    src.rows_cap = y_rows;
     if (tokens == 0) return ZBALHIP_OK;
     int threads = (int)((hidden / 8 + 63) / 64 * 64);
     if (threads > kThreads) threads = kThreads;
     hipStream_t st = (hipStream_t)stream;
     if (dtype == ZDT_BF16)
-        combine_kernel<ZDT_BF16><<<(unsigned)tokens, threads, 0, st>>>((const uint16_t *)y, base, base_is_inclusive, w,
-                                                                     topk_idx, send_token_idx, (int)hidden, (int)topk,
-                                                                     (int)experts, (uint16_t *)out);
+        combine_kernel<ZDT_BF16><<<(unsigned)tokens, threads, 0, st>>>(src, base, base_is_inclusive, w, topk_idx, send_token_idx,
+                                                                     (int)hidden, (int)topk, (int)experts, (uint16_t *)out);
     else
-        combine_kernel<ZDT_FP16><<<(unsigned)tokens, threads, 0, st>>>((const uint16_t *)y, base, base_is_inclusive, w,
-                                                                     topk_idx, send_token_idx, (int)hidden, (int)topk,
-                                                                     (int)experts, (uint16_t *)out);
+        combine_kernel<ZDT_FP16><<<(unsigned)tokens, threads, 0, st>>>(src, base, base_is_inclusive, w, topk_idx, send_token_idx,
+                                                                     (int)hidden, (int)topk, (int)experts, (uint16_t *)out);
     return zbalhip_check_launch();
 }

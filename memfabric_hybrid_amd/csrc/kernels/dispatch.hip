@@ -24,11 +24,28 @@ constexpr int kElemsPerLane = 16;
 
 enum { QM_COPY = 0, QM_INT8_EPS = 1, QM_FP8 = 2, QM_INT8_NOEPS = 3 };
 
-__device__ __forceinline__ int32_t pick_row(const int32_t *__restrict__ base, int base_inclusive, int e,
+/*
+ * Where the rows go. Expert e belongs to rank e / e_loc, whose receive window is dest[that rank] (and scale[that
+ * rank] for the quantisation scales); on one GPU the windows are local allocations, over xGMI they would be
+ * mapped peer memory, the kernel is the same. Offsets are looked up as base[e * ranks + my_rank]: the slot of
+ * this sender in the receiver's expert-major, then source-rank order (reference
+ * zbal_kernel_notify_dispatch.h:356-378, zbal_kernel_dispatch_normal.h:528-533). rows_cap is the number of rows
+ * each window holds; a pick that would land past it is dropped rather than written out of bounds.
+ */
+struct PeerRows {
+    uint8_t *dest[ZBALHIP_MAX_REDUCE_PEERS];
+    float *scale[ZBALHIP_MAX_REDUCE_PEERS];
+    int ranks, my_rank, e_loc;
+    int64_t rows_cap;
+};
+
+__device__ __forceinline__ int64_t pick_row(const int32_t *__restrict__ base, int base_inclusive, const PeerRows &pr, int e,
                                             int32_t rank_in_expert)
 {
-    const int32_t b = base_inclusive ? (e == 0 ? 0 : base[e - 1]) : base[e];
-    return b + rank_in_expert;
+    const int slot = e * pr.ranks + pr.my_rank;
+    const int32_t b = base_inclusive ? (slot == 0 ? 0 : base[slot - 1]) : base[slot];
+    const int64_t row = (int64_t)b + rank_in_expert;
+    return row < pr.rows_cap ? row : -1;
 }
 
 /* load 16 consecutive 16-bit elements as fp32 */
@@ -78,8 +95,7 @@ template <int XDT, int QM, int SLOTS, bool SMOOTH>
 __global__ void __launch_bounds__(kThreads)
 permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ topk_idx,
                      const int32_t *__restrict__ rank_in_expert, const int32_t *__restrict__ base, int base_inclusive,
-                     const float *__restrict__ smooth, int hidden, int topk, int experts, uint8_t *__restrict__ dest,
-                     float *__restrict__ dest_scale)
+                     const float *__restrict__ smooth, int hidden, int topk, int experts, PeerRows pr)
 {
     __shared__ float red[kThreads / 64];
     const int t = blockIdx.x;
@@ -115,7 +131,10 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             const int e = topk_idx[(int64_t)t * topk + k];
             const int rk = rank_in_expert[(int64_t)t * topk + k];
             if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
-            const int64_t row = pick_row(base, base_inclusive, e, rk);
+            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
+            if (row < 0) continue;
+            uint8_t *dest = pr.dest[e / pr.e_loc];
+            float *dest_scale = pr.scale[e / pr.e_loc];
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
                 const int seg = s * blockDim.x + threadIdx.x;
@@ -145,21 +164,25 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             const int e = topk_idx[(int64_t)t * topk + k];
             const int rk = rank_in_expert[(int64_t)t * topk + k];
             if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
-            const int64_t row = pick_row(base, base_inclusive, e, rk);
+            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
+            if (row < 0) continue;
+            uint8_t *dest = pr.dest[e / pr.e_loc];
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
                 const int seg = s * blockDim.x + threadIdx.x;
                 if (seg < nseg)
                     *reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16) = q[s];
             }
-            if (threadIdx.x == 0) dest_scale[row] = stored;
+            if (threadIdx.x == 0) pr.scale[e / pr.e_loc][row] = stored;
         }
     } else {
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
             const int rk = rank_in_expert[(int64_t)t * topk + k];
             if (e < 0 || e >= experts || rk < 0) continue; /* uniform across the block */
-            const int64_t row = pick_row(base, base_inclusive, e, rk);
+            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
+            if (row < 0) continue;
+            uint8_t *dest = pr.dest[e / pr.e_loc];
             float sv[SLOTS][16];
             float amax = 0.0f;
 #pragma unroll
@@ -184,7 +207,7 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
                     *reinterpret_cast<u32x4 *>(dest + row * hidden + (int64_t)seg * 16) = q;
                 }
             }
-            if (threadIdx.x == 0) dest_scale[row] = stored;
+            if (threadIdx.x == 0) pr.scale[e / pr.e_loc][row] = stored;
         }
     }
 }
@@ -193,7 +216,7 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
 __global__ void __launch_bounds__(kThreads)
 permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ topk_idx,
                     const int32_t *__restrict__ rank_in_expert, const int32_t *__restrict__ base, int base_inclusive,
-                    int hidden, int topk, int experts, uint16_t *__restrict__ dest)
+                    int hidden, int topk, int experts, PeerRows pr)
 {
     const int t = blockIdx.x;
     const int nchunk = hidden / 8;
@@ -208,7 +231,9 @@ permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ 
             const int e = topk_idx[(int64_t)t * topk + k];
             const int rk = rank_in_expert[(int64_t)t * topk + k];
             if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
-            const int64_t row = pick_row(base, base_inclusive, e, rk);
+            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
+            if (row < 0) continue;
+            uint16_t *dest = reinterpret_cast<uint16_t *>(pr.dest[e / pr.e_loc]);
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u * blockDim.x + threadIdx.x;
@@ -222,7 +247,7 @@ permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ 
 template <int XDT, int QM, bool SMOOTH>
 int32_t launch_quant(const void *x, const int32_t *topk_idx, const int32_t *rank_in_expert, const int32_t *base,
                      int base_inclusive, const float *smooth, int64_t tokens, int64_t hidden, int64_t topk,
-                     int64_t experts, void *dest, float *dest_scale, hipStream_t st)
+                     int64_t experts, const PeerRows &pr, hipStream_t st)
 {
     const int nseg = (int)(hidden / kElemsPerLane);
     int threads = (nseg + 63) / 64 * 64;
@@ -231,7 +256,7 @@ int32_t launch_quant(const void *x, const int32_t *topk_idx, const int32_t *rank
 #define ZB_LAUNCH(S)                                                                                              \
     permute_quant_kernel<XDT, QM, S, SMOOTH><<<(unsigned)tokens, threads, 0, st>>>(                                \
         (const uint16_t *)x, topk_idx, rank_in_expert, base, base_inclusive, smooth, (int)hidden, (int)topk,       \
-        (int)experts, (uint8_t *)dest, dest_scale)
+        (int)experts, pr)
     if (slots <= 1) ZB_LAUNCH(1);
     else if (slots <= 2) ZB_LAUNCH(2);
     else if (slots <= 4) ZB_LAUNCH(4);
@@ -244,12 +269,12 @@ int32_t launch_quant(const void *x, const int32_t *topk_idx, const int32_t *rank
 
 /*
  * Shared by the three public launchers. quant: QM_* flavour. `base` is the
- * exclusive (or inclusive) per-expert row offset table on the device.
+ * exclusive (or inclusive) per-expert row offset table on the device; `pr`
+ * says where each rank's rows go.
  */
-int32_t zbalhip_permute_internal(const void *x, int32_t x_dtype, const int32_t *topk_idx, const int32_t *rank_in_expert,
-                                 const int32_t *base, int base_inclusive, const float *smooth, int64_t tokens,
-                                 int64_t hidden, int64_t topk, int64_t experts, int quant, void *dest,
-                                 float *dest_scale, hipStream_t st)
+static int32_t permute_launch(const void *x, int32_t x_dtype, const int32_t *topk_idx, const int32_t *rank_in_expert,
+                              const int32_t *base, int base_inclusive, const float *smooth, int64_t tokens,
+                              int64_t hidden, int64_t topk, int64_t experts, int quant, const PeerRows &pr, hipStream_t st)
 {
     if (x_dtype != ZDT_BF16 && x_dtype != ZDT_FP16) return ZBALHIP_INVALID;
     if (hidden <= 0 || hidden > 16 * kThreads * 4 || topk <= 0 || tokens < 0) return ZBALHIP_INVALID;
@@ -257,18 +282,16 @@ int32_t zbalhip_permute_internal(const void *x, int32_t x_dtype, const int32_t *
     if (quant == QM_COPY) {
         if (hidden % 8 != 0) return ZBALHIP_INVALID;
         permute_copy_kernel<<<(unsigned)tokens, kThreads, 0, st>>>((const uint16_t *)x, topk_idx, rank_in_expert, base,
-                                                                 base_inclusive, (int)hidden, (int)topk, (int)experts,
-                                                                 (uint16_t *)dest);
+                                                                 base_inclusive, (int)hidden, (int)topk, (int)experts, pr);
         return zbalhip_check_launch();
     }
-    if (!dest_scale) return ZBALHIP_INVALID;
     if (hidden % 16 != 0 || (quant == QM_FP8 && hidden % 128 != 0)) return ZBALHIP_INVALID;
     const bool bf = (x_dtype == ZDT_BF16);
 #define ZB_GO(QMV, SM)                                                                                               \
     return bf ? launch_quant<ZDT_BF16, QMV, SM>(x, topk_idx, rank_in_expert, base, base_inclusive, smooth, tokens,  \
-                                                 hidden, topk, experts, dest, dest_scale, st)                        \
+                                                 hidden, topk, experts, pr, st)                                      \
               : launch_quant<ZDT_FP16, QMV, SM>(x, topk_idx, rank_in_expert, base, base_inclusive, smooth, tokens,  \
-                                                 hidden, topk, experts, dest, dest_scale, st)
+                                                 hidden, topk, experts, pr, st)
     if (quant == QM_FP8) { ZB_GO(QM_FP8, false); }
     if (quant == QM_INT8_EPS) { ZB_GO(QM_INT8_EPS, false); }
     if (quant == QM_INT8_NOEPS) {
@@ -279,16 +302,43 @@ int32_t zbalhip_permute_internal(const void *x, int32_t x_dtype, const int32_t *
     return ZBALHIP_INVALID;
 }
 
+/* one rank that owns every expert: all rows go to `dest` */
+static PeerRows single_window(void *dest, float *dest_scale, int64_t experts, int64_t rows_cap)
+{
+    PeerRows pr = {};
+    pr.dest[0] = (uint8_t *)dest;
+    pr.scale[0] = dest_scale;
+    pr.ranks = 1;
+    pr.my_rank = 0;
+    pr.e_loc = (int)experts;
+    pr.rows_cap = rows_cap;
+    return pr;
+}
+
 extern "C" int32_t zbalhip_dispatch_normal(const void *x, int32_t x_dtype, const int32_t *topk_idx,
                                            const int32_t *send_token_idx, const int32_t *put_offset, int64_t tokens,
                                            int64_t hidden, int64_t topk, int64_t experts, int32_t quant_mode,
-                                           void *dest, float *dest_scale, void *stream)
+                                           void *const *dest, float *const *dest_scale, int32_t ranks, int32_t my_rank,
+                                           int64_t dest_rows, void *stream)
 {
     if (!x || !topk_idx || !send_token_idx || !put_offset || !dest) return ZBALHIP_INVALID;
     if (experts <= 0 || quant_mode < 0 || quant_mode > 2) return ZBALHIP_INVALID;
+    if (ranks <= 0 || ranks > ZBALHIP_MAX_REDUCE_PEERS || my_rank < 0 || my_rank >= ranks || experts % ranks != 0 || dest_rows < 0)
+        return ZBALHIP_INVALID;
+    if (quant_mode != 0 && !dest_scale) return ZBALHIP_INVALID;
+    PeerRows pr = {};
+    for (int r = 0; r < ranks; ++r) {
+        if (!dest[r] || (quant_mode != 0 && !dest_scale[r])) return ZBALHIP_INVALID;
+        pr.dest[r] = (uint8_t *)dest[r];
+        pr.scale[r] = quant_mode != 0 ? dest_scale[r] : nullptr;
+    }
+    pr.ranks = ranks;
+    pr.my_rank = my_rank;
+    pr.e_loc = (int)(experts / ranks);
+    pr.rows_cap = dest_rows;
     const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_EPS : QM_FP8);
-    return zbalhip_permute_internal(x, x_dtype, topk_idx, send_token_idx, put_offset, 0, nullptr, tokens, hidden, topk,
-                                    experts, q, dest, dest_scale, (hipStream_t)stream);
+    return permute_launch(x, x_dtype, topk_idx, send_token_idx, put_offset, 0, nullptr, tokens, hidden, topk, experts, q, pr,
+                          (hipStream_t)stream);
 }
 
 extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, const int32_t *expert_ids,
@@ -298,8 +348,9 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
                                                 int32_t *ep_recv_counts, int32_t *scratch, int32_t scratch_blocks,
                                                 void *stream)
 {
-    if (!x || !expert_ids || !expand_x || !expand_idx || !expert_token_nums || !ep_recv_counts || !scratch)
-        return ZBALHIP_INVALID;
+    /* an empty batch has no per-token data: only the counts are written */
+    if (!expert_token_nums || !ep_recv_counts || !scratch) return ZBALHIP_INVALID;
+    if (tokens > 0 && (!x || !expert_ids || !expand_x || !expand_idx)) return ZBALHIP_INVALID;
     if (experts <= 0 || experts > 1024 || topk <= 0 || tokens < 0 || quant_mode < 0 || quant_mode > 2 ||
         scratch_blocks < 1)
         return ZBALHIP_INVALID;
@@ -308,8 +359,9 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
                                                      ep_recv_counts, nullptr, nullptr, expert_token_nums, st);
     if (rc != ZBALHIP_OK) return rc;
     const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_NOEPS : QM_FP8);
-    return zbalhip_permute_internal(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk,
-                                    experts, q, expand_x, dynamic_scales, st);
+    if (tokens > 0 && q != QM_COPY && !dynamic_scales) return ZBALHIP_INVALID;
+    return permute_launch(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk, experts, q,
+                          single_window(expand_x, dynamic_scales, experts, tokens * topk), st);
 }
 
 extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids,
@@ -319,7 +371,8 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
                                                int64_t *counts, int32_t *row_off, int32_t *scratch,
                                                int32_t scratch_blocks, void *stream)
 {
-    if (!x || !expert_ids || !q1 || !xs || !expand_idx || !counts || !row_off || !scratch) return ZBALHIP_INVALID;
+    if (!counts || !row_off || !scratch) return ZBALHIP_INVALID;
+    if (tokens > 0 && (!x || !expert_ids || !q1 || !xs || !expand_idx)) return ZBALHIP_INVALID;
     if (experts <= 0 || experts > 1024 || topk <= 0 || tokens < 0 || (mode != 1 && mode != 2) || scratch_blocks < 1)
         return ZBALHIP_INVALID;
     if (mode == 2 && smooth) return ZBALHIP_INVALID;
@@ -327,6 +380,6 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
     const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, 1, active_mask, expand_idx, nullptr,
                                                      row_off, counts, nullptr, st);
     if (rc != ZBALHIP_OK) return rc;
-    return zbalhip_permute_internal(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk,
-                                    experts, mode == 2 ? QM_FP8 : QM_INT8_NOEPS, q1, xs, st);
+    return permute_launch(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk, experts,
+                          mode == 2 ? QM_FP8 : QM_INT8_NOEPS, single_window(q1, xs, experts, tokens * topk), st);
 }

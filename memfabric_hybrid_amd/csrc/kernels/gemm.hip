@@ -644,7 +644,6 @@ grouped_gemm_dma_kernel(GemmParams p)
     while (true) {
         lid = next_id(lid);
         load_tile(lid, nxt);
-        if (nxt.valid) issue_sw(nxt, sw_buf ^ 1);   /* older than every slab issued below, so the slab waits cover it */
 
         f32x4 accf[4][8];
         i32x4 acci[4][8];
@@ -677,6 +676,12 @@ grouped_gemm_dma_kernel(GemmParams p)
                 wait_vmcnt<0>();
             }
             __syncthreads();                /* slab kb has landed for everybody; the stage read in the step before is free */
+            /*
+             * The next tile's weight block scales go into the buffer the tile before this one used. Every wave is
+             * past this tile's first barrier now, so none of them still reads that buffer; the transfers are older
+             * than every slab issued from here on, so the slab waits cover them.
+             */
+            if (kb == 0 && nxt.valid) issue_sw(nxt, sw_buf ^ 1);
             /*
              * That stage takes the slab NSTAGE-1 steps ahead, which may belong to the next tile. It is issued in parts,
              * spread over the first half of this step's MFMAs: a wave that pushes all of its loads at once sits in the

@@ -313,6 +313,67 @@ layout_scan_kernel(const int32_t *__restrict__ hist, int nblk, int experts, int 
     }
 }
 
+/*
+ * Notify for a group of R ranks, from the point of view of rank `me` (reference zbal_kernel_notify_dispatch.h
+ * ReorderRecvDataOutput :356-378, BuildTotalRecvTokens :531-564, BuildRecvTokenPerExp :566-596,
+ * BuildBalanceMatrix :421-498 without re-balancing). counts.p[s] is rank s's tokens-per-expert vector, read where
+ * it lies in that rank's window. For every destination rank r the offsets are the exclusive running sum of
+ * counts[s][r * E_loc + le] taken local expert by local expert and, within an expert, source rank by source rank.
+ * One block, one thread per (local expert, source rank) pair of a destination rank.
+ */
+struct CountsOfRanks {
+    const int32_t *p[ZBALHIP_MAX_REDUCE_PEERS];
+};
+
+__global__ void __launch_bounds__(ZB_MAX_EXPERTS)
+notify_ranks_kernel(CountsOfRanks counts, int ranks, int me, int experts, int topk, int32_t *__restrict__ recv_data,
+                    int32_t *__restrict__ put_offset, int32_t *__restrict__ total_recv,
+                    int64_t *__restrict__ recv_tokens_per_expert, int32_t *__restrict__ balance)
+{
+    __shared__ int32_t wsum[ZB_MAX_EXPERTS / 64];
+    __shared__ int32_t rank_total[ZBALHIP_MAX_REDUCE_PEERS];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int e_loc = experts / ranks;
+    for (int i = tid; i < ranks * experts; i += blockDim.x) recv_data[i] = counts.p[i / experts][i % experts];
+    if (tid < ranks) rank_total[tid] = 0;
+    __syncthreads();
+    for (int r = 0; r < ranks; ++r) {
+        const int le = tid / ranks, s = tid - le * ranks;
+        const int32_t c = tid < experts ? counts.p[s][r * e_loc + le] : 0;
+        int32_t incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int32_t o = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += o;
+        }
+        if (lane == 63) wsum[wave] = incl;
+        __syncthreads();
+        int32_t add = 0, all = 0;
+        for (int w = 0; w < nwaves; ++w) {
+            if (w < wave) add += wsum[w];
+            all += wsum[w];
+        }
+        if (tid < experts) put_offset[r * experts + tid] = incl + add - c;
+        if (r == me && tid == 0) *total_recv = all;
+        /* what source rank s sends in all: the sum over destination ranks of its share */
+        if (tid < experts && c) atomicAdd(&rank_total[s], c);
+        __syncthreads();
+    }
+    for (int le = tid; le < e_loc; le += blockDim.x) {
+        int64_t sum = 0;
+        for (int s = 0; s < ranks; ++s) sum += counts.p[s][me * e_loc + le];
+        recv_tokens_per_expert[le] = sum;
+    }
+    for (int i = tid; i < ranks * 2 * ranks; i += blockDim.x) {
+        const int row = i / (2 * ranks), col = i - row * 2 * ranks;
+        const int32_t bs = rank_total[row] / topk;
+        int32_t v = -1;
+        if (bs > 0 && col == 2 * row) v = 0;
+        if (bs > 0 && col == 2 * row + 1) v = bs - 1;
+        balance[i] = v;
+    }
+}
+
 /* ---- router ----------------------------------------------------------------- */
 
 /*
@@ -518,13 +579,26 @@ extern "C" int32_t zbalhip_dispatch_layout_static(const void *topk_idx, int32_t 
                                  nullptr, nullptr, nullptr, (hipStream_t)stream);
 }
 
-extern "C" int32_t zbalhip_dispatch_notify(const int32_t *tokens_per_expert, int64_t experts, int64_t topk,
-                                           int32_t *recv_data, int32_t *put_offset, int32_t *total_recv,
-                                           int64_t *recv_tokens_per_expert, int32_t *balance_matrix, void *stream)
+extern "C" int32_t zbalhip_dispatch_notify(const int32_t *const *tokens_per_expert, int32_t ranks, int32_t my_rank,
+                                           int64_t experts, int64_t topk, int32_t *recv_data, int32_t *put_offset,
+                                           int32_t *total_recv, int64_t *recv_tokens_per_expert, int32_t *balance_matrix,
+                                           void *stream)
 {
     if (!tokens_per_expert || !recv_data || !put_offset || !total_recv || !recv_tokens_per_expert || !balance_matrix)
         return ZBALHIP_INVALID;
     if (experts <= 0 || experts > ZB_MAX_EXPERTS || topk <= 0) return ZBALHIP_INVALID;
-    return zbalhip_scan_internal(tokens_per_expert, 0, experts, topk, 1, recv_data, put_offset, nullptr, nullptr,
-                                 recv_tokens_per_expert, nullptr, total_recv, balance_matrix, (hipStream_t)stream);
+    if (ranks <= 0 || ranks > ZBALHIP_MAX_REDUCE_PEERS || my_rank < 0 || my_rank >= ranks || experts % ranks != 0)
+        return ZBALHIP_INVALID;
+    for (int r = 0; r < ranks; ++r)
+        if (!tokens_per_expert[r]) return ZBALHIP_INVALID;
+    if (ranks == 1)
+        return zbalhip_scan_internal(tokens_per_expert[0], 0, experts, topk, 1, recv_data, put_offset, nullptr, nullptr,
+                                     recv_tokens_per_expert, nullptr, total_recv, balance_matrix, (hipStream_t)stream);
+    CountsOfRanks counts = {};
+    for (int r = 0; r < ranks; ++r) counts.p[r] = tokens_per_expert[r];
+    const int threads = (int)((experts + 63) / 64 * 64);
+    notify_ranks_kernel<<<1, threads, 0, (hipStream_t)stream>>>(counts, ranks, my_rank, (int)experts, (int)topk, recv_data,
+                                                                put_offset, total_recv, recv_tokens_per_expert,
+                                                                balance_matrix);
+    return zbalhip_check_launch();
 }

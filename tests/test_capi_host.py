@@ -205,3 +205,20 @@ def test_fused_workspace_size_is_monotonic(lib):
     assert f(128, 7168, 8, 32, 4096, 4096, 0) == a
     assert f(128, 7168, 1, 32, 512, 4096, 0) > f(128, 7168, 1, 32, 512, 0, 0)
     assert f(128, 7168, 8, 32, 4096, 100, 0) == 0
+
+
+def test_kernel_seam_types_and_exports():
+    """CommGroupInfo keeps the reference's layout (zbal_comm_host_device_struct.h:133-151: 2160 bytes,
+    peerGroupRank2WorldRank at 64) and the nine launcher functions of zbal_npu_operators.h are exported with C++
+    linkage."""
+    import ctypes
+    assert ctypes.sizeof(capi.CommGroupInfo) == 2160
+    assert capi.CommGroupInfo.peerGroupRank2WorldRank.offset == 64
+    assert capi.CommGroupInfo.localDeviceMemSize.offset == 2112
+    assert capi.CommGroupInfo.waitSymbol.offset == 2120
+    assert capi.CommGroupInfo.groupIndex.offset == 2152
+    names = set(capi.cxx_symbols())
+    assert names == {"ZBALOpReduceScatter", "ZBALOpAllReduce", "ZBALOpDispatchLayout", "ZBALOpNotifyDispatch",
+                     "ZBALOpDispatchNormal", "ZBALOpCombineNormal", "ZBALOpDispatchLowLatency", "ZBALOpCombineLowLatency",
+                     "ZBALOpFusedDeepMoe"}
+    assert set(capi.CXX_SIGNATURES) <= names

@@ -530,6 +530,36 @@ def test_fused_moe_active_mask(buf, mode, active):
         assert np.array_equal(got[:active], ref)
 
 
+@pytest.mark.parametrize("active", [0, 23, 70])
+def test_fused_moe_shared_expert_with_active_mask(buf, active):
+    """Shared expert and x_active_mask together: the shared expert, too, sees only the first sum(mask) tokens
+    (the reference processes nothing past them, TokenActiveMaskCal ...swiglu_quant_multistage_workspace.h:836-863);
+    the other rows of both outputs keep what they held."""
+    T, H, K, E, I, mode = 70, 256, 4, 8, 128, 0
+    x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 160)
+    _, _, _, sw1, ss1, sw2, ss2 = fused_inputs(T, H, 1, 1, 256, mode, 161)
+    mask = np.zeros(T, dtype=bool)
+    mask[:active] = True
+    seven = lambda: torch.full((T, H), 7.0, dtype=torch.bfloat16, device="cuda")
+    pack = lambda w: buf.prepack_weight(dev(w))
+    out, share, nums = buf.fused_deep_moe(
+        dev(x, torch.bfloat16), dev(ids), pack(w1), dev(s1), pack(w2), dev(s2, torch.bfloat16), dev(es), E, quant_mode=mode,
+        share_gmm1_weight=pack(sw1), share_gmm1_scale=dev(ss1), share_gmm2_weight=pack(sw2),
+        share_gmm2_scale=dev(ss2, torch.bfloat16), x_active_mask=dev(mask), out=seven(), share_out=seven())
+    untouched = host(torch.full((T - active, H), 7.0, dtype=torch.bfloat16))
+    assert np.array_equal(host(out)[active:], untouched)
+    assert np.array_equal(host(share)[active:], untouched)
+    if active == 0:
+        assert not host(nums).any()
+        return
+    ref, counts = zo.fused_moe(x[:active], zo.DT_BF16, ids[:active], es[:active], w1, s1, w2, s2, E, mode)
+    ref_share, _ = zo.fused_moe(x[:active], zo.DT_BF16, np.zeros((active, 1), np.int64), np.ones((active, 1), np.float32),
+                                sw1, ss1, sw2, ss2, 1, mode)
+    assert np.array_equal(host(nums), counts)
+    assert np.array_equal(host(out)[:active], ref)
+    assert np.array_equal(host(share)[:active], ref_share)
+
+
 @pytest.mark.parametrize("mode", [0, 2, 3])
 @pytest.mark.parametrize("T", [70, 700])
 def test_fused_moe_tensor_list_weights(buf, mode, T):
