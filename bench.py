@@ -351,7 +351,7 @@ def bench_reduce(args, torch, np, capi, buf):
         # a one-input "reduction" is a plain copy of known traffic (2 x 256 MiB): the calibration point for
         # the FETCH_SIZE / WRITE_SIZE counters
         arr = (ctypes.c_void_p * 1)(peers[1].data_ptr())
-        capi.check("copy", lib.zbalhip_reduce(arr, 1, n, zdt, capi.REDUCE_SUM, out.data_ptr(), 0, st))
+        capi.check("copy", lib.zbalhip_reduce(arr, 1, n, zdt, capi.REDUCE_SUM, out.data_ptr(), 0, None, 0, st))
         torch.cuda.synchronize()
         del peers, out, ref
     destroy_group(comm)

@@ -149,9 +149,9 @@ ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype,
  * constant 100 MHz clock. Workgroup b < ZBALHIP_TRACE_UNITS of a traced kernel
  * writes to block b (one lane, begin and end of each frame); a block that is
  * full drops further records.
- *   zbalhip_trace_alloc: pinned, zeroed host memory and its device address.
- *   zbalhip_trace_configure: the ring that kernels launched from now on write
- *     to (null = tracing off, the state at start-up). One ring per process.
+ *   zbalhip_trace_alloc: pinned, zeroed host memory and its device address;
+ *     the owner (a communicator) passes that address to the launches it wants
+ *     traced, so every communicator has a ring of its own.
  *   zbalhip_trace_sync: waits until the device is idle, so that the ring holds
  *     every record of the kernels launched so far.
  *   zbalhip_trace_free: waits for the device, then releases the memory.
@@ -162,7 +162,6 @@ ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype,
 #define ZBALHIP_TRACE_FRAME_SHIFT 56
 #define ZBALHIP_TRACE_BE_SHIFT 62
 ZBALHIP_API int32_t zbalhip_trace_alloc(int64_t points, uint64_t **host_ring, uint64_t **device_ring);
-ZBALHIP_API int32_t zbalhip_trace_configure(uint64_t *device_ring, int64_t points);
 ZBALHIP_API int32_t zbalhip_trace_sync(void);
 ZBALHIP_API int32_t zbalhip_trace_free(uint64_t *host_ring);
 
@@ -175,10 +174,11 @@ ZBALHIP_API int32_t zbalhip_trace_free(uint64_t *host_ring);
  * op is a zbal_reduce_op_t value; PROD is a true product. trace_frame != 0
  * (a zbal_profiling_name_t value of the reference,
  * zbal_comm_host_device_struct.h:27-70) records that frame around each traced
- * workgroup's work when a trace ring is configured.
+ * workgroup's work in `trace_ring` (device address from zbalhip_trace_alloc,
+ * `trace_points` words per block; null = not traced).
  */
 ZBALHIP_API int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t count, int32_t dtype, int32_t op, void *out,
-                       int32_t trace_frame, void *stream);
+                       int32_t trace_frame, uint64_t *trace_ring, int64_t trace_points, void *stream);
 
 /* p[0..n) = value, as a kernel (safe to record into a HIP graph, unlike a memset node) */
 ZBALHIP_API int32_t zbalhip_fill_i32(int32_t *p, int64_t n, int32_t value, void *stream);

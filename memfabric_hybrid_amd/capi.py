@@ -126,9 +126,8 @@ SIGNATURES = {
     "zbalhip_combine": (_i32, [_vp, _i32, _i32, _i64, _i32, _vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _vp, _vp]),
     "zbalhip_dispatch_low_latency": (_i32, [_vp, _i32, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp,
                                             _vp, _vp, _i32, _vp]),
-    "zbalhip_reduce": (_i32, [ctypes.POINTER(_vp), _i32, _i64, _i32, _i32, _vp, _i32, _vp]),
+    "zbalhip_reduce": (_i32, [ctypes.POINTER(_vp), _i32, _i64, _i32, _i32, _vp, _i32, _vp, _i64, _vp]),
     "zbalhip_trace_alloc": (_i32, [_i64, ctypes.POINTER(ctypes.POINTER(ctypes.c_uint64)), ctypes.POINTER(ctypes.POINTER(ctypes.c_uint64))]),
-    "zbalhip_trace_configure": (_i32, [ctypes.POINTER(ctypes.c_uint64), _i64]),
     "zbalhip_trace_sync": (_i32, []),
     "zbalhip_trace_free": (_i32, [ctypes.POINTER(ctypes.c_uint64)]),
     "zbalhip_weight_prepack": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp]),

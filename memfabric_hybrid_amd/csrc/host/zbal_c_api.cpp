@@ -125,7 +125,7 @@ ZBAL_API int32_t zbal_comm_register_peer_window(zbal_comm_t comm, uint16_t rank,
     ZBAL_VALIDATE_RETURN(rank < c->Info().groupSize, "RegisterPeerWindow failed as rank " << rank << " is out of range", Z_INVALID_PARAM);
     ZBAL_VALIDATE_RETURN(base != nullptr && size > 0, "RegisterPeerWindow failed as the window is empty", Z_INVALID_PARAM);
     ZBAL_VALIDATE_RETURN((reinterpret_cast<uintptr_t>(base) & 15u) == 0, "RegisterPeerWindow failed as the window is not 16-byte aligned", Z_INVALID_PARAM);
-    c->MutableInfo().peers[rank] = PeerWindow{base, size};
+    c->RegisterPeer(rank, PeerWindow{base, size});
     return Z_OK;
 }
 

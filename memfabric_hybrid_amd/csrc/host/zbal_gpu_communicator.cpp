@@ -92,8 +92,8 @@ public:
      * Tracing follows the reference's switches (zbal_env_helper.h:20-22, SetupProfMemory
      * zbal_npu_communicator_base.cpp:145-199): ZBAL_PROF_ENABLE=1 turns it on, ZBAL_PROF_MAX_TRACING_COUNT is the
      * number of 64-bit words per traced workgroup (20480 unless in [20480, 204800)), ZBAL_PROF_DIR the directory
-     * of the dump. The ring is pinned host memory the kernels write directly. The process has one active ring:
-     * the one of the communicator created last with tracing on.
+     * of the dump. The ring is pinned host memory the kernels write directly; every communicator created with
+     * tracing on owns one and hands it to its own launches.
      */
     explicit GpuCommunicator(const GroupInfo &info) : Communicator(info)
     {
@@ -110,14 +110,12 @@ public:
             return;
         }
         tracePoints_ = points;
-        zbalhip_trace_configure(traceDev_, tracePoints_);
     }
 
     ~GpuCommunicator() override
     {
         if (traceHost_ == nullptr) return;
         DumpProfilingTrace();
-        zbalhip_trace_configure(nullptr, 0);
         zbalhip_trace_free(traceHost_);
     }
 
@@ -190,14 +188,15 @@ public:
                 out[r] = static_cast<const uint8_t *>(p) + ((int64_t)info_.worldRank[r] - me) * (int64_t)info_.peerStride;
             return true;
         }
-        const PeerWindow &mine = info_.peers[info_.myGroupRank];
+        const std::vector<PeerWindow> peers = Peers();
+        const PeerWindow &mine = peers[info_.myGroupRank];
         const uintptr_t a = reinterpret_cast<uintptr_t>(p), b = reinterpret_cast<uintptr_t>(mine.base);
         if (mine.base == nullptr || a < b || a + bytes > b + mine.size) {
             ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as the send buffer is not inside this rank's registered window");
             return false;
         }
         for (uint16_t r = 0; r < info_.groupSize; ++r) {
-            const PeerWindow &w = info_.peers[r];
+            const PeerWindow &w = peers[r];
             if (w.base == nullptr || (a - b) + bytes > w.size) {
                 ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as rank " << r << " has no window covering the buffer");
                 return false;
@@ -210,7 +209,7 @@ public:
     /* the copies of `p` in every rank's window; a group of one needs no window: its only copy is `p` itself */
     bool PeerCopies(const char *op, const void *p, size_t bytes, const void **out) const
     {
-        if (info_.groupSize == 1 && info_.peerStride == 0 && info_.peers[0].base == nullptr) {
+        if (info_.groupSize == 1 && info_.peerStride == 0 && Peers()[0].base == nullptr) {
             out[0] = p;
             return true;
         }
@@ -245,14 +244,15 @@ public:
         }
         const size_t es = ElemSize(dt);
         const void *peer[ZBALHIP_MAX_REDUCE_PEERS];
-        if (info_.groupSize == 1 && info_.peerStride == 0 && info_.peers[0].base == nullptr) {
+        if (info_.groupSize == 1 && info_.peerStride == 0 && Peers()[0].base == nullptr) {
             peer[0] = send; /* a group of one needs no window */
         } else if (!Translate(opName, send, (sliceOffsetElems + count) * es, peer)) {
             return Z_INVALID_PARAM;
         }
         for (uint16_t r = 0; r < info_.groupSize; ++r)
             peer[r] = static_cast<const uint8_t *>(peer[r]) + sliceOffsetElems * es;
-        return Launched(opName, zbalhip_reduce(peer, info_.groupSize, (int64_t)count, dt, op, recv, traceFrame, stream));
+        return Launched(opName, zbalhip_reduce(peer, info_.groupSize, (int64_t)count, dt, op, recv, traceFrame, traceDev_,
+                                               tracePoints_, stream));
     }
 
     int32_t AllReduce(const void *send, void *recv, void *, size_t count, zbal_datatype_t dt, zbal_reduce_op_t op,

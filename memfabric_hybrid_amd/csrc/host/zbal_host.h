@@ -128,7 +128,18 @@ public:
     /* writes what the device trace ring holds as a trace-viewer file; a no-op when tracing is off
        (reference zbal_communicator.h:114) */
     virtual void DumpProfilingTrace() noexcept {}
-    GroupInfo &MutableInfo() { return info_; }
+
+    /* peer windows may be registered while another thread runs an operator on the same communicator */
+    void RegisterPeer(uint16_t rank, const PeerWindow &w)
+    {
+        std::lock_guard<std::mutex> guard(peersMutex_);
+        info_.peers[rank] = w;
+    }
+    std::vector<PeerWindow> Peers() const
+    {
+        std::lock_guard<std::mutex> guard(peersMutex_);
+        return info_.peers;
+    }
 
     virtual int32_t AllReduce(const void *send, void *recv, void *buffer, size_t count, zbal_datatype_t dt,
                               zbal_reduce_op_t op, aclrtStream stream) = 0;
@@ -189,6 +200,7 @@ public:
 
 protected:
     GroupInfo info_;
+    mutable std::mutex peersMutex_;
 };
 
 using CommunicatorPtr = std::shared_ptr<Communicator>;
@@ -207,6 +219,8 @@ zbal_comm_t ByName(const std::string &name);
 /* shared ownership keeps the object alive for the duration of an operator call */
 CommunicatorPtr Find(zbal_comm_t comm);
 uint32_t Count();
+/* every communicator writes its device trace (reference Communicator::DumpAllComm, zbal_communicator.cpp:180-186) */
+void DumpAllTraces();
 } // namespace registry
 
 /* Layout of the fused operator's workspace; one function so that sizing and carving cannot diverge. */

@@ -176,5 +176,15 @@ uint32_t Count()
     return (uint32_t)gByName.size();
 }
 
+void DumpAllTraces()
+{
+    std::vector<CommunicatorPtr> all;
+    {
+        std::lock_guard<std::mutex> guard(gMutex);
+        for (auto &kv : gByName) all.push_back(kv.second);
+    }
+    for (auto &c : all) c->DumpProfilingTrace();
+}
+
 } // namespace registry
 } // namespace zbal

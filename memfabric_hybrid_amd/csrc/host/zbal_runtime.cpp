@@ -6,6 +6,7 @@
  * and no symmetric heap, peers being windows registered per communicator.
  */
 #include <atomic>
+#include <csignal>
 #include <cstdio>
 #include <cstring>
 
@@ -52,6 +53,12 @@ BootState &Boot()
 } // namespace zbal
 
 using namespace zbal;
+
+/* SIGUSR1 writes every communicator's device trace, as in the reference (common/zbal_signal_handler.cpp:21-29) */
+static void DumpTracesOnSignal(int sig)
+{
+    if (sig == SIGUSR1) registry::DumpAllTraces();
+}
 
 /* the kernel launchers' way to leave a last-error text (declared in kernels/zbal_device.h) */
 void zbalhip_set_last_error(const char *text) { ZBAL_LOG_AND_SET_LAST_ERROR(text); }
@@ -121,6 +128,7 @@ __attribute__((visibility("default"))) int32_t zbal_bootstrap(zbal_bootstrap_opt
         ZBAL_VALIDATE_RETURN(e == hipSuccess, "Bootstrap failed as hipSetDevice failed: " << hipGetErrorString(e),
                              Z_INIT_BOOTSTRAP_FAILED);
     }
+    std::signal(SIGUSR1, DumpTracesOnSignal); /* installed by bootstrap, reference bootstrap/zbal_bootstrap_default.cpp:102 */
     st.bootstrapped = true;
     st.worldSize = options->worldSize;
     st.rankId = options->rankId;

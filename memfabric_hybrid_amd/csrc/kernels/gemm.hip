@@ -30,6 +30,7 @@
  * the workgroups resident on an XCD share both their A and their W slabs in
  * that XCD's L2.
  */
+#include <mutex>
 #include <type_traits>
 
 #include "zbal_device.h"
@@ -896,19 +897,30 @@ template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
 int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
 {
     using S = DmaShape<TM, NSTAGE, MODE == MODE_W4A8 ? 64 : 128>;
+    static std::mutex mu;          /* one per kernel instantiation: guards its per-device set-up below */
     static int cus[64] = {};
     const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE>);
-    int dev = 0;
+    int dev = 0, n_cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ZBALHIP_RT_ERROR;
-    if (cus[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return ZBALHIP_RT_ERROR;
-        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
-            return ZBALHIP_RT_ERROR;
-        cus[dev] = n;
+    {
+        std::lock_guard<std::mutex> guard(mu);
+        if (cus[dev] == 0) {
+            /* the first launch on a device raises the kernel's LDS limit, which cannot be recorded into a graph */
+            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+            if (st != nullptr && hipStreamIsCapturing(st, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone) {
+                zbalhip_set_last_error("grouped GEMM: the first launch on a device must happen outside of a stream capture");
+                return ZBALHIP_RT_ERROR;
+            }
+            int n = 0;
+            if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return ZBALHIP_RT_ERROR;
+            if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
+                return ZBALHIP_RT_ERROR;
+            cus[dev] = n;
+        }
+        n_cus = cus[dev];
     }
     unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, TM);
-    const unsigned resident = (unsigned)(cus[dev] + 7) / 8 * 8;
+    const unsigned resident = (unsigned)(n_cus + 7) / 8 * 8;
     if (grid > resident) grid = resident;
     grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE><<<grid, S::THREADS, S::LDS_BYTES, st>>>(p);
     return zbalhip_check_launch();

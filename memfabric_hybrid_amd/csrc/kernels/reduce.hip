@@ -21,10 +21,6 @@ struct ReducePtrs {
     uint32_t trace_frame;
 };
 
-/* the process's trace ring: what zbalhip_trace_configure set last */
-unsigned long long *g_trace_ring = nullptr;
-uint32_t g_trace_points = 0;
-
 /*
  * One record into this workgroup's block of the ring (reference ZBAL_PROF_RECORD, zbal_kernel_trace.h:22-42):
  * bump the block's index word, then write the record there. Called by one lane of workgroups below
@@ -253,14 +249,6 @@ extern "C" int32_t zbalhip_trace_alloc(int64_t points, uint64_t **host_ring, uin
     return ZBALHIP_OK;
 }
 
-extern "C" int32_t zbalhip_trace_configure(uint64_t *device_ring, int64_t points)
-{
-    if (device_ring != nullptr && (points <= ZBALHIP_TRACE_REC_OFF || points > (1 << 24))) return ZBALHIP_INVALID;
-    g_trace_ring = (unsigned long long *)device_ring;
-    g_trace_points = device_ring ? (uint32_t)points : 0;
-    return ZBALHIP_OK;
-}
-
 extern "C" int32_t zbalhip_trace_sync(void) { return hipDeviceSynchronize() == hipSuccess ? ZBALHIP_OK : ZBALHIP_RT_ERROR; }
 
 extern "C" int32_t zbalhip_trace_free(uint64_t *host_ring)
@@ -271,14 +259,15 @@ extern "C" int32_t zbalhip_trace_free(uint64_t *host_ring)
 }
 
 extern "C" int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t count, int32_t dtype, int32_t op,
-                                  void *out, int32_t trace_frame, void *stream)
+                                  void *out, int32_t trace_frame, uint64_t *trace_ring, int64_t trace_points, void *stream)
 {
     if (!in || !out || n_in <= 0 || n_in > ZBALHIP_MAX_REDUCE_PEERS || count <= 0) return ZBALHIP_INVALID;
     if (trace_frame < 0 || trace_frame >= (1 << (ZBALHIP_TRACE_BE_SHIFT - ZBALHIP_TRACE_FRAME_SHIFT))) return ZBALHIP_INVALID;
+    if (trace_ring != nullptr && (trace_points <= ZBALHIP_TRACE_REC_OFF || trace_points > (1 << 24))) return ZBALHIP_INVALID;
     ReducePtrs ptrs;
     for (int p = 0; p < ZBALHIP_MAX_REDUCE_PEERS; ++p) ptrs.p[p] = p < n_in ? in[p] : nullptr;
-    ptrs.trace = trace_frame ? g_trace_ring : nullptr;
-    ptrs.trace_points = g_trace_points;
+    ptrs.trace = trace_frame ? (unsigned long long *)trace_ring : nullptr;
+    ptrs.trace_points = trace_ring ? (uint32_t)trace_points : 0;
     ptrs.trace_frame = (uint32_t)trace_frame;
     /* the vector path needs 16-byte aligned bases */
     bool aligned = ((uintptr_t)out & 15u) == 0;

@@ -238,7 +238,7 @@ def test_reduce_kernel_all_types(buf, dt, op):
         d_in = [dev(a, tdt) for a in ins]
         out = torch.empty_like(d_in[0])
         arr = (ctypes.c_void_p * N)(*[t.data_ptr() for t in d_in])
-        assert lib.zbalhip_reduce(arr, N, n, dt, op, out.data_ptr(), 0, capi.stream_ptr()) == 0
+        assert lib.zbalhip_reduce(arr, N, n, dt, op, out.data_ptr(), 0, None, 0, capi.stream_ptr()) == 0
         ref = zo.reduce(ins, dt, op)
         assert np.array_equal(host(out), ref), (N, n)
 
@@ -254,7 +254,7 @@ def test_reduce_full_size_sampled_windows(buf):
         ins = [torch.randn(n, device="cuda", generator=g).to(tdt) for _ in range(N)]
         out = torch.empty_like(ins[0])
         arr = (ctypes.c_void_p * N)(*[t.data_ptr() for t in ins])
-        assert lib.zbalhip_reduce(arr, N, n, dt, capi.REDUCE_SUM, out.data_ptr(), 0, capi.stream_ptr()) == 0
+        assert lib.zbalhip_reduce(arr, N, n, dt, capi.REDUCE_SUM, out.data_ptr(), 0, None, 0, capi.stream_ptr()) == 0
         torch.cuda.synchronize()
         w = 1 << 16
         for start in [0, n - w] + [int(v) for v in rng(6).integers(0, n - w, 6)]:
@@ -349,6 +349,20 @@ def test_device_trace_ring_and_trace_viewer_dump(buf, tmp_path, monkeypatch):
             ts = [e["ts"] for e in mine]
             assert all(b <= a for b, a in zip(ts, ts[1:]))
             assert ts[-1] - ts[0] < 5e6                                        # microseconds: the launches took well under 5 s
+        # SIGUSR1 dumps every communicator's trace (reference common/zbal_signal_handler.cpp:21-29)
+        import os, signal
+        for f in files:
+            os.remove(f)
+        os.kill(os.getpid(), signal.SIGUSR1)
+        assert len(glob.glob(str(tmp_path / "trace_view_1_*.json"))) == 1
+        # a second traced communicator has a ring of its own: destroying it leaves this one's tracing on
+        other = create_group("traced_other", 1, 0)
+        destroy_group(other)
+        assert lib.zbal_reduce_scatter(wins[me].data_ptr(), recv.data_ptr(), n, capi.DT_BF16, capi.REDUCE_SUM, comm,
+                                       capi.stream_ptr()) == 0
+        assert lib.zbal_comm_dump_profiling_trace(comm) == 0
+        newest = max(glob.glob(str(tmp_path / "trace_view_1_*.json")), key=os.path.getmtime)
+        assert len([e for e in json.load(open(newest)) if e["name"] == "RS_KERNEL_ALL"]) == 2 * (launches + 1) * wgs
     finally:
         torch.cuda.synchronize()
         destroy_group(comm)
