@@ -195,8 +195,9 @@ ZO_API void zo_set_num_threads(int32_t n)
 /*
  * Router. parity unpinned: the reference has none; its tests draw
  * topk_idx with torch.topk and weights at random (test_low_latency.py:68-89).
- * Definition: p = softmax(logits) in fp32 (max-subtracted, glibc expf, sum in
- * index order); the K picks are the K largest logits, ties to the lower
+ * Definition: p = softmax(logits) in fp32 (max-subtracted; exp is the fixed
+ * polynomial zo_expf_impl that the GPU router evaluates too, pinned against
+ * the float64 exp to 2.5e-7; sum in index order); the K picks are the K largest logits, ties to the lower
  * index, listed in descending order; w_k = p_k / sum of the K picked p.
  * Pinned by brute force and by invariants in the tests.
  */
@@ -209,7 +210,7 @@ ZO_API void zo_topk_route(const float *logits, int64_t T, int64_t E, int64_t K, 
         for (int64_t e = 1; e < E; ++e) mx = std::max(mx, l[e]);
         std::vector<float> p(E);
         float sum = 0.0f;
-        for (int64_t e = 0; e < E; ++e) { p[e] = expf(l[e] - mx); sum += p[e]; }
+        for (int64_t e = 0; e < E; ++e) { p[e] = zo_expf_impl(l[e] - mx); sum += p[e]; }
         for (int64_t e = 0; e < E; ++e) p[e] = p[e] / sum;
         std::vector<char> used(E, 0);
         float wsum = 0.0f;

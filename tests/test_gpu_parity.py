@@ -34,7 +34,7 @@ def test_router(buf, T, E, K):
     idx, w = buf.topk_route(dev(logits), K)
     ridx, rw = zo.topk_route(logits, K)
     assert np.array_equal(host(idx), ridx)
-    assert np.allclose(host(w), rw, rtol=2e-6, atol=0)     # north star: weights within 1e-6 relative (2 ulp slack)
+    assert np.allclose(host(w), rw, rtol=1e-6, atol=0)     # north star: weights within 1e-6 relative
 
 
 # ---- layout / notify -------------------------------------------------------------------------

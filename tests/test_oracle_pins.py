@@ -77,7 +77,7 @@ def test_router_brute_force_and_invariants():
         order = sorted(range(E), key=lambda e: (-logits[t, e], e))[:K]
         assert list(idx[t]) == order
         ref = p[t, order] / p[t, order].sum()
-        assert np.allclose(w[t], ref, rtol=2e-6, atol=0)
+        assert np.allclose(w[t], ref, rtol=1e-6, atol=0)
     assert np.allclose(w.sum(1), 1.0, atol=1e-6)
     assert list(idx[4]) == [0, 1]
 
@@ -432,3 +432,98 @@ def test_reduce_bf16_single_rounding():
     h = [zo.f32_to_fp16(b) for b in bufs32[:2]]
     o = zo.reduce(h, zo.DT_FP16, 1)
     assert np.array_equal(o, (h[0].view(np.float16).astype(np.float32) + h[1].view(np.float16).astype(np.float32)).astype(np.float16).view(np.uint16))
+
+
+# ---- branch-level pins: smooth scales, all-zero rows, the fused permute, integer wrap-around, half max/min/prod ----
+
+def _np_quant_int8_noeps(v):
+    """numpy float32 restatement of the eps-less per-token quantisation: s = 127/amax, q = rint(v*s), scale = 1/s;
+    an all-zero row gives q = 0, scale = 0. Every product is rounded to float32, as separate operations."""
+    amax = np.abs(v).max()
+    if amax == 0:
+        return np.zeros(v.shape, np.int8), np.float32(0)
+    s = np.float32(127.0) / amax
+    q = np.clip(np.rint((v * s).astype(np.float32)), -128, 127).astype(np.int8)
+    return q, np.float32(1.0) / s
+
+
+def test_fused_permute_quant_rows_smooth_scales_and_zero_rows():
+    T, H, K, E = 37, 256, 3, 6
+    g = rng(200)
+    xf = g.standard_normal((T, H)).astype(np.float32) * 3
+    xf[5] = 0.0                                   # an all-zero token: q = 0, scale = 0 (no division by zero)
+    x = zo.f32_to_bf16(xf)
+    xv = zo.bf16_to_f32(x)
+    ids = g.integers(-1, E + 1, size=(T, K)).astype(np.int32)      # some ids invalid
+    smooth = g.uniform(0.25, 2.0, (E, H)).astype(np.float32)
+    smooth[2, :] = 0.0                            # smoothing can zero a row too
+    for sm in (None, smooth):
+        q1, xs, eidx, counts = zo.fused_permute_quant(x, zo.DT_BF16, ids, sm, E, 1)
+        # permutation: expert-major, flat-pick order inside an expert (numpy stable sort of the valid picks)
+        flat = ids.reshape(-1)
+        valid = np.flatnonzero((flat >= 0) & (flat < E))
+        order = valid[np.argsort(flat[valid], kind="stable")]
+        assert np.array_equal(counts, np.bincount(flat[valid], minlength=E))
+        assert q1.shape[0] == len(order)
+        for row, pick in enumerate(order):
+            t, e = pick // K, flat[pick]
+            v = xv[t] if sm is None else (xv[t] * sm[e]).astype(np.float32)
+            q, sc = _np_quant_int8_noeps(v)
+            assert np.array_equal(q1[row], q), (row, t, e)
+            assert xs[row].view(np.uint32) == sc.view(np.uint32), (row, t, e)
+            assert eidx.reshape(-1)[pick] == np.sum(flat[:pick] == e)
+        assert np.all(eidx.reshape(-1)[(flat < 0) | (flat >= E)] == -1)
+        zero_rows = [r for r, pick in enumerate(order) if pick // K == 5 or (sm is not None and flat[pick] == 2)]
+        assert zero_rows and all(xs[r] == 0 and not q1[r].any() for r in zero_rows)
+
+
+def test_fused_permute_quant_fp8_rows_match_torch_cast():
+    T, H, K, E = 19, 256, 2, 4
+    g = rng(201)
+    x = zo.f32_to_bf16(g.standard_normal((T, H)).astype(np.float32))
+    xv = zo.bf16_to_f32(x)
+    ids = g.integers(0, E, size=(T, K)).astype(np.int32)
+    q1, xs, _, _ = zo.fused_permute_quant(x, zo.DT_BF16, ids, None, E, 2)
+    flat = ids.reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    for row, pick in enumerate(order):
+        v = xv[pick // K].reshape(H // 128, 128)
+        amax = np.maximum(np.abs(v).max(1), np.float32(1e-4))
+        scaled = (v * (np.float32(448.0) / amax)[:, None]).astype(np.float32)
+        want = torch.from_numpy(np.clip(scaled, -448, 448)).to(torch.float8_e4m3fn).view(torch.uint8).numpy().reshape(-1)
+        assert np.array_equal(q1[row], want)
+        assert np.array_equal(xs[row].view(np.uint32), (amax * np.float32(1.0 / 448.0)).astype(np.float32).view(np.uint32))
+
+
+@pytest.mark.parametrize("dt,npdt", [(0, np.int8), (1, np.int16), (3, np.int64)])
+def test_reduce_integers_wrap_around(dt, npdt):
+    info = np.iinfo(npdt)
+    g = rng(210 + dt)
+    bufs = [g.integers(info.min, info.max, 2000, dtype=npdt, endpoint=True) for _ in range(6)]
+    with np.errstate(over="ignore"):
+        s = bufs[0].copy()
+        p = bufs[0].copy()
+        for b in bufs[1:]:
+            s = (s + b).astype(npdt)              # numpy integer arithmetic is modular
+            p = (p * b).astype(npdt)
+    assert np.array_equal(zo.reduce(bufs, dt, 1), s)
+    assert np.array_equal(zo.reduce(bufs, dt, 0), p)
+    assert np.array_equal(zo.reduce(bufs, dt, 2), np.max(np.stack(bufs), 0))
+    assert np.array_equal(zo.reduce(bufs, dt, 3), np.min(np.stack(bufs), 0))
+    # the exact sum modulo 2^bits, computed with Python integers
+    bits = info.bits
+    exact = [(sum(int(b[i]) for b in bufs) + (1 << (bits - 1))) % (1 << bits) - (1 << (bits - 1)) for i in range(50)]
+    assert list(zo.reduce(bufs, dt, 1)[:50]) == exact
+
+
+@pytest.mark.parametrize("dt,to16,from16", [(zo.DT_BF16, zo.f32_to_bf16, zo.bf16_to_f32), (zo.DT_FP16, zo.f32_to_fp16, zo.fp16_to_f32)])
+def test_reduce_halves_max_min_prod(dt, to16, from16):
+    g = rng(220)
+    bufs = [to16(g.uniform(0.5, 1.5, 3000).astype(np.float32) * g.choice([-1.0, 1.0], 3000).astype(np.float32)) for _ in range(5)]
+    vals = np.stack([from16(b) for b in bufs])
+    assert np.array_equal(zo.reduce(bufs, dt, 2), to16(vals.max(0)))          # max / min of representable values: no rounding
+    assert np.array_equal(zo.reduce(bufs, dt, 3), to16(vals.min(0)))
+    acc = vals[0].copy()
+    for v in vals[1:]:
+        acc = (acc * v).astype(np.float32)        # fp32 running product in buffer order, one rounding at the end
+    assert np.array_equal(zo.reduce(bufs, dt, 0), to16(acc))

@@ -57,3 +57,30 @@ def max_rel_err(got, want):
     got = got.astype(np.float64)
     want = want.astype(np.float64)
     return float(np.abs(got - want).max() / max(np.abs(want).max(), 1e-30))
+
+
+def elem_rel_err(got, want, floor_frac=1.0 / 64):
+    """max |got - want| / |want| over the elements whose reference magnitude is at least floor_frac of the largest
+    one: the element-wise companion of max_rel_err (which divides every difference by the largest magnitude)."""
+    got = got.astype(np.float64)
+    want = want.astype(np.float64)
+    big = np.abs(want) >= floor_frac * max(np.abs(want).max(), 1e-30)
+    return float((np.abs(got - want)[big] / np.abs(want)[big]).max()) if big.any() else 0.0
+
+
+FP8_GEMM_ELEM_TOL = 1.6e-2      # two bf16 roundings of slack on a single GEMM output element
+
+
+def assert_fp8_close(got, want, what="", elem_tol=None):
+    """The bar for the block-scaled fp8 path: max error relative to the largest magnitude below 2e-2 (the stated
+    tolerance). elem_tol adds an element-wise bound over the elements of appreciable size (>= 1/64 of the largest):
+    used for single GEMMs, where the only difference from the oracle is the summation order inside a 128-deep
+    block. A whole layer is not held to it: the re-quantisation between the GEMMs can move an intermediate to the
+    neighbouring e4m3 code (a 2^-4 step), and the weighted combine cancels, so single small outputs may differ by
+    tens of per cent while the layer agrees to 1e-4 in the reference's calc_diff. Returns both figures."""
+    g, w = got.astype(np.float64), want.astype(np.float64)
+    e_max, e_elem = max_rel_err(g, w), elem_rel_err(g, w)
+    assert e_max < 2e-2, "%s: max error relative to the largest magnitude %.3g" % (what, e_max)
+    if elem_tol is not None:
+        assert e_elem < elem_tol, "%s: element-wise relative error %.3g" % (what, e_elem)
+    return e_max, e_elem
