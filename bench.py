@@ -58,6 +58,9 @@ def parse():
                     help="prefill = the headline fp8 MoE layer (default); decode = 128-token W8A8 layer with Zipf routing; "
                          "qwen_w4a8 = 16384-token W4A8 layer; reduce = the 8 x 256 MiB local reduction")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--equal-rows", action="store_true",
+                    help="profiling only (prefill): token t picks experts (t*topk + j) mod experts, so every expert receives "
+                         "exactly tokens*topk/experts rows; the figure says what the ragged row counts of random routing cost")
     ap.add_argument("--no-others", action="store_true",
                     help="headline workload only: leave out the `other_workloads` block (reduce, decode, W4A8)")
     return ap.parse_args()
@@ -152,7 +155,11 @@ def bench_moe(args, torch, np, capi, buf, workload):
     rows = T * K
     torch.manual_seed(0)
     x = torch.randn((T, H), device=dev, dtype=torch.float32).to(torch.bfloat16)
-    if cfg["zipf"] is None:
+    if workload == "prefill" and args.equal_rows:
+        picks = (torch.arange(T, device=dev)[:, None] * K + torch.arange(K, device=dev)[None, :]) % E
+        logits = torch.rand((T, E), device=dev, dtype=torch.float32)
+        logits.scatter_add_(1, picks, torch.ones((T, K), device=dev))
+    elif cfg["zipf"] is None:
         logits = torch.rand((T, E), device=dev, dtype=torch.float32)          # uniform-random logits
     else:
         # Zipf(s) popularity over a fixed random permutation of the experts; adding Gumbel noise to log p makes
@@ -261,7 +268,7 @@ def bench_moe(args, torch, np, capi, buf, workload):
         roofline = {"kernel": kname, "bound": "mfma", "achieved": flops1 / t1 / 1e12,
                     "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s" if mode == 2 else "TOP/s",
                     "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
-                    "traffic": GMM1_TRAFFIC_BYTES_T4096 if (workload == "prefill" and T == 4096) else None}
+                    "traffic": GMM1_TRAFFIC_BYTES_T4096 if (workload == "prefill" and T == 4096 and not args.equal_rows) else None}
     stages = {
         "ms": {k: round(v, 4) for k, v in stage_ms.items()},
         "gmm1_tflops": flops1 / t1 / 1e12,
@@ -309,7 +316,9 @@ def bench_moe(args, torch, np, capi, buf, workload):
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
         "config": {"workload": cfg["name"], "tokens": T, "hidden": H, "experts": E, "topk": K, "intermediate": I,
-                   "quant": cfg["quant"], "parallelism": "1 GPU", "l2_flush_between_steps": False},
+                   "quant": cfg["quant"], "parallelism": "1 GPU", "l2_flush_between_steps": False,
+                   "routing": "equal rows per expert (profiling)" if (workload == "prefill" and args.equal_rows) else
+                              ("uniform-random logits" if cfg["zipf"] is None else "Zipf(%.1f) popularity" % cfg["zipf"])},
         "roofline": roofline, "cpu_baseline": cpu, "stages": stages, "parity": parity,
     }
     return line
