@@ -76,7 +76,7 @@ def main():
     import numpy as np
     import torch
     from memfabric_hybrid_amd import capi
-    from memfabric_hybrid_amd.buffer import Buffer
+    from memfabric_hybrid_amd.operators import OperatorBuffer as Buffer
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
@@ -327,7 +327,7 @@ def bench_moe(args, torch, np, capi, buf, workload):
 def bench_reduce(args, torch, np, capi, buf):
     """BASELINE configs[3]: one rank's reduce-scatter shard, 8 peer buffers of 256 MiB held as local HBM
     allocations, through zbal_reduce_scatter. Algorithmic bytes = (8 + 1) x 256 MiB = 2.416 GB per launch."""
-    from memfabric_hybrid_amd.buffer import create_group, destroy_group
+    from memfabric_hybrid_amd.operators import create_group, destroy_group
     lib = buf.lib
     R, nbytes = 8, 256 << 20
     comm = create_group("bench_rs8", R, 0)

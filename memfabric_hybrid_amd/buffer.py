@@ -1,313 +1,372 @@
-"""Host-side mirror of the reference's DeepEP-compatible adaptor for one rank.
+"""DeepEP-compatible `Buffer` for one MI355X: the Python face a caller of the reference switches to.
 
-`Buffer` follows adaptor::deep_ep::Buffer (reference
-app/zbal/src/csrc/adaptor/deepep/zbal_deepep.cpp) and its Python face
-(app/zbal/src/python/zbal/zbal_buffer.py): the same method names, the same
-tensors allocated with the same shapes and dtypes, each method one or more
-calls through the zbal C ABI. Differences, all deliberate:
-  * no host synchronisation between notify and dispatch (the reference reads
-    the received-token count back with .item(), zbal_deepep.cpp:359): outputs
-    are sized for the worst case tokens * topk rows;
-  * one process: MoE operators run on a group of one rank; further "ranks" exist only as HBM windows
-    for the reductions;
-  * `use_fp8` selects real e4m3 with 1x128 scales when fp8_block_scale=True
-    (the reference maps the flag to int8, zbal_deepep.cpp:514,525).
-torch is used for device memory and streams only.
+Method names, positional order, defaults and return tuples follow the reference's
+`zbal.Buffer` (app/zbal/src/python/zbal/zbal_buffer.py) and the C++ adaptor under it
+(app/zbal/src/csrc/adaptor/deepep/zbal_deepep.cpp); each method cites the lines it
+mirrors. The work is done by `operators.OperatorBuffer` (kept as `self.runtime`, the
+name the reference gives its C++ object), which calls the zbal C ABI.
+
+What differs, because this build runs one rank on one GPU:
+  * `group` may be None (or any object with rank() / size()); a group of more than one
+    rank is refused: the cross-rank transport is not part of this build;
+  * `fused_deep_moe` takes the weights in the operator's logical layout
+    ([experts, hidden, gmm1_h_len] and [experts, gmm1_h_len / 2, hidden]) exactly as the
+    reference does before its NZ format cast (test/python/deepep/test_fused_deep_moe.py:66-69)
+    and pre-packs them once per weight tensor (cached); already pre-packed tensors from
+    `prepack_weight` pass through;
+  * `dispatch` honours `num_worst_tokens` (no host synchronisation, empty list), which
+    the reference accepts and ignores;
+  * events are real: `EventOverlap.current_stream_wait()` waits for the stream position
+    captured when the operator returned (the reference's is a no-op).
 """
-import ctypes
 import os
-import threading
+from typing import Callable, List, Optional, Tuple, Union
 
 import torch
 
 from . import capi
-
-_LOCK = threading.Lock()
-_STATE = {"world": None, "local": None, "users": 0}
-
-# The process models this many "ranks" as local HBM windows; reductions may use groups up to this size.
-MODEL_WORLD_SIZE = 16
+from .operators import OperatorBuffer
 
 
-def _create_comm(lib, name, world, size, rank):
-    co = capi.CommOptions(name=name, backendType=capi.BACKEND_GPU, isWorldGroup=world, groupSize=size,
-                          groupRankId=rank)
-    comm = ctypes.c_void_p()
-    capi.check("zbal_comm_create", lib.zbal_comm_create(ctypes.byref(co), ctypes.byref(comm)))
-    return comm
+class Config:
+    """Tuning record of the reference (adaptor/deepep/zbal_deepep_config.h:23-49); the kernels here take no tuning."""
+
+    def __init__(self, num_sms: int, num_max_nvl_chunked_send_tokens: int, num_max_nvl_chunked_recv_tokens: int,
+                 num_max_rdma_chunked_send_tokens: int, num_max_rdma_chunked_recv_tokens: int) -> None:
+        self.num_sms = num_sms
+        self.num_max_nvl_chunked_send_tokens = num_max_nvl_chunked_send_tokens
+        self.num_max_nvl_chunked_recv_tokens = num_max_nvl_chunked_recv_tokens
+        self.num_max_rdma_chunked_send_tokens = num_max_rdma_chunked_send_tokens
+        self.num_max_rdma_chunked_recv_tokens = num_max_rdma_chunked_recv_tokens
+
+    def get_nvl_buffer_size_hint(self, hidden_bytes: int, num_ranks: int) -> int:
+        return hidden_bytes
+
+    def get_rdma_buffer_size_hint(self, hidden_bytes: int, num_ranks: int) -> int:
+        return hidden_bytes
 
 
-def _acquire(device_index):
-    """Bootstrap once per process; returns the one-rank group the MoE operators run on."""
-    lib = capi.load()
-    with _LOCK:
-        if _STATE["world"] is None:
-            opts = capi.BootstrapOptions()
-            capi.check("zbal_bootstrap_options_init", lib.zbal_bootstrap_options_init(ctypes.byref(opts)))
-            opts.worldSize, opts.rankId, opts.deviceId = MODEL_WORLD_SIZE, 0, device_index
-            capi.check("zbal_bootstrap", lib.zbal_bootstrap(ctypes.byref(opts), None))
-            _STATE["world"] = _create_comm(lib, b"world", 1, MODEL_WORLD_SIZE, 0)
-            _STATE["local"] = _create_comm(lib, b"local", 0, 1, 0)
-        _STATE["users"] += 1
-        return _STATE["local"]
+class EventHandle:
+    """A position on the current stream (adaptor/deepep/zbal_deep_event.h:22-31, there without content)."""
+
+    def __init__(self) -> None:
+        self.event = torch.cuda.Event()
+        self.event.record(torch.cuda.current_stream())
+
+    def current_stream_wait(self) -> None:
+        torch.cuda.current_stream().wait_event(self.event)
 
 
-def _release():
-    lib = capi.load()
-    with _LOCK:
-        _STATE["users"] -= 1
-        if _STATE["users"] == 0 and _STATE["world"] is not None:
-            lib.zbal_comm_destroy_all(0)
-            lib.zbal_unbootstrap(0)
-            _STATE["world"] = _STATE["local"] = None
+class EventOverlap:
+    """python/zbal/zbal_utils.py:8-36: an event plus tensors kept alive until it has passed."""
+
+    def __init__(self, event: Optional[EventHandle] = None, extra_tensors: Optional[Tuple[torch.Tensor]] = None) -> None:
+        self.event = event
+        self.extra_tensors = extra_tensors
+
+    def current_stream_wait(self) -> None:
+        if self.event is not None:
+            self.event.current_stream_wait()
 
 
-def create_group(name, size, rank):
-    """A sub-group of `size` modelled ranks in which this process is `rank` (needs a live Buffer)."""
-    if _STATE["world"] is None:
-        raise RuntimeError("create a Buffer first: it bootstraps the library")
-    return _create_comm(capi.load(), name.encode(), 0, size, rank)
+def get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
+                                   num_experts: int) -> int:
+    """adaptor/deepep/zbal_deepep_config.cpp:18-24."""
+    return num_max_dispatch_tokens_per_rank
 
 
-def destroy_group(comm):
-    capi.check("zbal_comm_destroy", capi.load().zbal_comm_destroy(comm, 0))
+PADDING_SIZE = 1      # an empty batch is padded to this many tokens (zbal_deepep.cpp:85, 470-490)
 
 
 class Buffer:
-    """One-rank MoE dispatch / combine / fused-MoE buffer (DeepEP-style interface)."""
+    """zbal_buffer.py:12-84. One rank, one GPU: dispatch and combine permute through this GPU's HBM."""
 
-    num_ranks = 1
-    rank = 0
+    num_sms: int = 20
 
-    def __init__(self, device=None):
-        if not torch.cuda.is_available():
-            raise RuntimeError("memfabric_hybrid_amd.Buffer needs a GPU; there is no CPU path")
-        self.device = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
-        self.lib = capi.load()
-        self.comm = _acquire(self.device.index or 0)
-        self.send_token_idx = None       # kept between layout, dispatch and combine (zbal_deepep.cpp:254,305,423)
-        self._tables = {}                # device address tables of tensor-list operands
-        self._closed = False
+    def __init__(self, group=None, num_nvl_bytes: int = 0, num_rdma_bytes: int = 0, low_latency_mode: bool = False,
+                 num_qps_per_rank: int = 12, allow_nvlink_for_low_latency_mode: bool = True,
+                 allow_mnnvl: bool = False, device=None) -> None:
+        self.rank = group.rank() if group is not None else 0
+        self.group_size = group.size() if group is not None else 1
+        if self.group_size != 1:
+            raise NotImplementedError("this build runs the MoE operators on a group of one rank (one GPU)")
+        self.num_nvl_bytes = num_nvl_bytes
+        self.num_rdma_bytes = num_rdma_bytes
+        self.low_latency_mode = low_latency_mode
+        self.runtime = OperatorBuffer(device)
+        self.device = self.runtime.device
+        self._packed = {}          # logical weight tensor -> its pre-packed copy
+        self._pad = None           # what low_latency_dispatch padded, for the combine that follows
 
-    def close(self):
-        if not self._closed:
-            self._closed = True
-            _release()
+    def close(self) -> None:
+        self.runtime.close()
 
-    def __del__(self):
-        try:
-            self.close()
-        except Exception:
-            pass
-
-    # -- helpers ---------------------------------------------------------------------------
-    def _empty(self, shape, dtype):
-        return torch.empty(shape, dtype=dtype, device=self.device)
+    # ---- static helpers -------------------------------------------------------------------------------
+    @staticmethod
+    def get_dispatch_config(num_ranks: int) -> Config:
+        """zbal_buffer.py:86-109 (the table's one-rank entry is this build's addition)."""
+        table = {1: (24, 256, 6, 128), 2: (24, 256, 6, 128), 4: (6, 256, 6, 128), 8: (6, 256, 6, 128),
+                 16: (36, 288, 20, 128), 24: (8, 288, 32, 128), 32: (32, 288, 32, 128), 64: (20, 288, 28, 128),
+                 128: (20, 560, 32, 128), 144: (32, 720, 12, 128), 160: (28, 720, 12, 128)}
+        return Config(Buffer.num_sms, *table[num_ranks])
 
     @staticmethod
-    def _ti(t, **kw):
-        return ctypes.byref(capi.tensor_info(t, **kw))
+    def get_combine_config(num_ranks: int) -> Config:
+        """zbal_buffer.py:111-135."""
+        table = {1: (10, 256, 6, 128), 2: (10, 256, 6, 128), 4: (9, 256, 6, 128), 8: (4, 256, 6, 128),
+                 16: (4, 288, 12, 128), 24: (1, 288, 8, 128), 32: (1, 288, 8, 128), 64: (1, 288, 20, 128),
+                 128: (1, 560, 12, 128), 144: (2, 720, 8, 128), 160: (2, 720, 8, 128)}
+        return Config(Buffer.num_sms, *table[num_ranks])
 
-    def _list_ti(self, seq, num_experts, **kw):
-        """Descriptor of a tensor list: shape and type of the stacked tensor, `data` = a device table of the
-        per-expert addresses (kept in a small cache, so repeated calls with the same tensors copy nothing)."""
-        if len(seq) != num_experts:
-            raise ValueError("a tensor list needs one tensor per expert")
-        first = seq[0]
-        per = tuple(first.shape[1:]) if first.shape[0] == 1 and first.dim() == 3 else tuple(first.shape)
-        for t in seq:
-            if not t.is_contiguous() or t.dtype != first.dtype or t.numel() != first.numel():
-                raise ValueError("tensor-list entries must be contiguous and alike")
-        key = tuple(t.data_ptr() for t in seq)
-        table = self._tables.get(key)
-        if table is None:
-            if len(self._tables) >= 64:
-                self._tables.clear()
-            table = torch.tensor(key, dtype=torch.int64).to(self.device)
-            self._tables[key] = table
-        ti = capi.tensor_info(first, shape=(num_experts,) + per, **kw)
-        ti.data = table.data_ptr()
-        return ctypes.byref(ti)
+    @staticmethod
+    def set_num_sms(new_num_sms: int) -> None:
+        """zbal_buffer.py:137-146."""
+        if not new_num_sms % 2 == 0:
+            raise ValueError("The SM count must be even")
+        Buffer.num_sms = new_num_sms
 
-    # -- router (extension) ------------------------------------------------------------------
-    def topk_route(self, logits, num_topk, idx_dtype=torch.int64):
-        """idx_dtype: torch.int64 (what get_dispatch_layout takes) or torch.int32 (what dispatch / fused_deep_moe take)"""
-        T = logits.shape[0]
-        idx = self._empty((T, num_topk), idx_dtype)
-        w = self._empty((T, num_topk), torch.float32)
-        capi.check("zbal_moe_topk_route", self.lib.zbal_moe_topk_route(
-            self._ti(logits), num_topk, self._ti(idx), self._ti(w), self.comm, capi.stream_ptr(), 0))
-        return idx, w
+    @staticmethod
+    def capture() -> EventOverlap:
+        """zbal_buffer.py:148-155: an event on the current stream."""
+        return EventOverlap(EventHandle())
 
-    # -- normal mode -------------------------------------------------------------------------
-    def get_dispatch_layout(self, topk_idx, num_experts):
-        """zbal_deepep.cpp:209-257. Returns (num_tokens_per_rank, None, num_tokens_per_expert, is_token_in_rank, None)."""
-        assert topk_idx.dim() == 2 and topk_idx.is_contiguous() and topk_idx.dtype == torch.int64
-        T, K = topk_idx.shape
-        per_expert = self._empty((num_experts,), torch.int32)
-        per_rank = self._empty((self.num_ranks,), torch.int32)
-        send_idx = self._empty((T, K), torch.int32)
-        scratch = self._empty((num_experts * 50,), torch.int32)
-        capi.check("zbal_dispatch_normal_layout", self.lib.zbal_dispatch_normal_layout(
-            self._ti(topk_idx), T, num_experts, K, self._ti(per_rank), self._ti(per_expert), self._ti(send_idx),
-            self._ti(scratch), self.comm, capi.stream_ptr(), 0))
-        self.send_token_idx = send_idx
-        valid = (topk_idx >= 0) & (topk_idx < num_experts)
-        is_token_in_rank = valid.any(dim=1, keepdim=True).to(torch.int32)   # the reference leaves this unwritten
-        return per_rank, None, per_expert, is_token_in_rank, None
+    @staticmethod
+    def get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank: int, hidden: int, num_ranks: int,
+                                       num_experts: int) -> int:
+        """zbal_buffer.py:157-166."""
+        return get_low_latency_rdma_size_hint(num_max_dispatch_tokens_per_rank, hidden, num_ranks, num_experts)
 
-    def dispatch(self, x, topk_idx, topk_weights, num_tokens_per_expert, quant_mode=capi.NO_QUANT):
-        """zbal_deepep.cpp:259-393. Returns (recv_x, recv_x_scales, num_recv_tokens_per_expert (device int64), handle)."""
-        assert self.send_token_idx is not None, "call get_dispatch_layout first"
-        T, H = x.shape
-        K = topk_idx.shape[1]
-        E = num_tokens_per_expert.shape[0]
-        expert_ids = topk_idx.to(torch.int32)
-        recv_data = self._empty((1, E), torch.int32)
-        recv_per_expert = self._empty((E,), torch.int64)
-        put_offset = self._empty((1, E), torch.int32)
-        balance = self._empty((1, 2), torch.int32)
-        total = self._empty((1,), torch.int32)
-        st = capi.stream_ptr()
-        capi.check("zbal_dispatch_normal_notify", self.lib.zbal_dispatch_normal_notify(
-            self._ti(num_tokens_per_expert), E, K, self._ti(recv_data), self._ti(total), self._ti(recv_per_expert),
-            self._ti(put_offset), self._ti(balance), self.comm, st, 0))
-        rows = max(T * K, 1)
-        if quant_mode == capi.NO_QUANT:
-            recv_x = self._empty((rows, H), x.dtype)
-            scales = self._empty((1,), torch.float32)
-        elif quant_mode == capi.QUANT_INT8:
-            recv_x = self._empty((rows, H), torch.int8)
-            scales = self._empty((rows,), torch.float32)
-        else:
-            recv_x = self._empty((rows, H), torch.float8_e4m3fn)
-            scales = self._empty((rows, H // 128), torch.float32)
-        capi.check("zbal_dispatch_normal", self.lib.zbal_dispatch_normal(
-            self._ti(x), self._ti(expert_ids), self._ti(self.send_token_idx), self._ti(put_offset), self._ti(balance),
-            E, quant_mode, self._ti(recv_x), self._ti(scales), self.comm, st, 0))
-        handle = dict(put_offset=put_offset, balance_matrix=balance, expert_ids=expert_ids,
-                      send_token_idx=self.send_token_idx, total_recv=total, num_experts=E)
-        return recv_x, scales, recv_per_expert, handle
+    @staticmethod
+    def _wait(previous_event: Optional[EventOverlap]) -> None:
+        if previous_event is not None:
+            previous_event.current_stream_wait()
 
-    def combine(self, x, handle, topk_weights):
-        """zbal_deepep.cpp:395-452."""
-        T, K = handle["expert_ids"].shape
-        H = x.shape[1]
-        out = self._empty((T, H), x.dtype)
-        capi.check("zbal_combine_normal", self.lib.zbal_combine_normal(
-            self._ti(x), self._ti(handle["put_offset"]), self._ti(topk_weights), self._ti(handle["expert_ids"]),
-            self._ti(handle["send_token_idx"]), self._ti(handle["balance_matrix"]), handle["num_experts"],
-            self._ti(out), self.comm, capi.stream_ptr(), 0))
-        return out
+    @staticmethod
+    def _event(async_finish: bool, tensors=None) -> EventOverlap:
+        return EventOverlap(EventHandle(), tensors) if async_finish else EventOverlap(None)
 
-    # -- low-latency mode ----------------------------------------------------------------------
-    def low_latency_dispatch(self, x, topk_idx, num_max_dispatch_tokens_per_rank, num_experts, use_fp8=True,
-                             fp8_block_scale=False):
-        """zbal_deepep.cpp:454-565. Returns (packed_recv_x, packed_recv_x_scales, packed_recv_count, handle)."""
-        T, H = x.shape
-        K = topk_idx.shape[1]
-        expert_ids = topk_idx.to(torch.int32)
-        rows = max(T * K, 1)
+    # ---- normal mode ----------------------------------------------------------------------------------
+    def get_dispatch_layout(self, topk_idx: torch.Tensor, num_experts: int,
+                            previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
+                            allocate_on_comm_stream: bool = False
+                            ) -> Tuple[torch.Tensor, Optional[torch.Tensor], torch.Tensor, torch.Tensor, EventOverlap]:
+        """zbal_buffer.py:168-214, zbal_deepep.cpp:209-257. topk_idx [tokens, topk] int64, -1 = no selection.
+        Returns (num_tokens_per_rank, None, num_tokens_per_expert, is_token_in_rank, event)."""
+        if topk_idx.dim() != 2 or not topk_idx.is_contiguous():
+            raise ValueError("Layout: topk_idx must be a contiguous [num_tokens, num_topk] tensor")
+        if num_experts <= 0:
+            raise ValueError("Layout: check num_experts failed: %d" % num_experts)
+        self._wait(previous_event)
+        per_rank, per_rdma, per_expert, in_rank, _ = self.runtime.get_dispatch_layout(topk_idx, num_experts)
+        return per_rank, per_rdma, per_expert, in_rank, self._event(async_finish)
+
+    def dispatch(self, x: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]], handle: Optional[Tuple] = None,
+                 num_tokens_per_rank: Optional[torch.Tensor] = None,
+                 num_tokens_per_rdma_rank: Optional[torch.Tensor] = None,
+                 is_token_in_rank: Optional[torch.Tensor] = None,
+                 num_tokens_per_expert: Optional[torch.Tensor] = None, topk_idx: Optional[torch.Tensor] = None,
+                 topk_weights: Optional[torch.Tensor] = None, expert_alignment: int = 1, num_worst_tokens: int = 0,
+                 config: Optional[Config] = None, previous_event: Optional[EventOverlap] = None,
+                 async_finish: bool = False, allocate_on_comm_stream: bool = False,
+                 dispatch_wait_recv_cost_stats: Optional[torch.Tensor] = None
+                 ) -> Tuple[Union[Tuple[torch.Tensor, torch.Tensor], torch.Tensor], Optional[torch.Tensor],
+                            Optional[torch.Tensor], List[int], Tuple, EventOverlap]:
+        """zbal_buffer.py:216-348, zbal_deepep.cpp:259-393. Rows arrive expert-major, in flat pick order within an
+        expert. With DEEP_NORMAL_MODE_USE_INT8_QUANT=1 the rows are int8 with one fp32 scale each and recv_x is the
+        pair. Like the reference this reads the received-row count back (one host synchronisation) to size recv_x
+        and to build the Python list, unless num_worst_tokens is given: then recv_x has that many rows, the list is
+        empty and nothing waits for the GPU.
+        Returns (recv_x, None, None, num_recv_tokens_per_expert_list, handle, event)."""
+        config = self.get_dispatch_config(self.group_size) if config is None else config
+        if isinstance(x, tuple):
+            raise NotImplementedError("Not support fp8")
+        use_quant = os.getenv("DEEP_NORMAL_MODE_USE_INT8_QUANT") == "1"
+        if handle is not None:
+            raise NotImplementedError("Optional communication handle is not supported yet.")
+        if not (num_tokens_per_rank is not None and is_token_in_rank is not None and num_tokens_per_expert is not None):
+            raise ValueError("num_tokens_per_rank, is_token_in_rank, num_tokens_per_expert must be valid")
+        if num_tokens_per_expert.dtype != torch.int32 or num_tokens_per_rank.dtype != torch.int32:
+            raise ValueError("num_tokens_per_expert and num_tokens_per_rank must be torch.int")
+        if x.dim() != 2 or not x.is_contiguous():
+            raise ValueError("x dim not 2 or not contiguous")
+        if num_tokens_per_expert.dim() != 1 or num_tokens_per_expert.size(0) % self.group_size != 0:
+            raise ValueError("num_tokens_per_expert check failed")
+        if num_tokens_per_rank.dim() != 1 or num_tokens_per_rank.size(0) != self.group_size:
+            raise ValueError("num_tokens_per_rank check failed")
+        if topk_idx is None or topk_idx.dim() != 2 or topk_idx.size(0) != x.size(0) or not topk_idx.is_contiguous():
+            raise ValueError("topk_idx check failed")
         token_nums_type = int(os.environ.get("MOE_EXPERT_TOKEN_NUMS_TYPE", "1"))
-        if not use_fp8:
-            qm, recv = capi.NO_QUANT, self._empty((rows, H), x.dtype)
-            scales = self._empty((rows,), torch.float32)
-        elif fp8_block_scale:
-            qm, recv = capi.QUANT_FP8_B128, self._empty((rows, H), torch.float8_e4m3fn)
-            scales = self._empty((rows, H // 128), torch.float32)
+        if token_nums_type not in (0, 1):
+            raise ValueError("expert_token_nums_type is invalid")
+        self._wait(previous_event)
+        K = topk_idx.size(1)
+        note = self.runtime.notify(num_tokens_per_expert, K)
+        counts = None
+        if num_worst_tokens > 0:
+            rows = num_worst_tokens
         else:
-            qm, recv = capi.QUANT_INT8, self._empty((rows, H), torch.int8)
-            scales = self._empty((rows,), torch.float32)
-        expand_idx = self._empty((rows,), torch.int32)
-        ep_recv_count = self._empty((num_experts,), torch.int32)
-        packed_recv_count = self._empty((num_experts,), torch.int64)
-        put_offset = self._empty((num_experts,), torch.int32)
-        put_offset_status = self._empty((num_experts,), torch.float32)
-        capi.check("zbal_dispatch_low_latency", self.lib.zbal_dispatch_low_latency(
-            self._ti(x), self._ti(expert_ids), num_experts, 1, 0, qm, max(T, num_max_dispatch_tokens_per_rank), 0,
-            token_nums_type, self._ti(recv), self._ti(scales), self._ti(expand_idx), self._ti(packed_recv_count),
-            self._ti(ep_recv_count), self._ti(put_offset), self._ti(put_offset_status), self.comm, capi.stream_ptr(),
-            0))
-        handle = dict(expert_ids=expert_ids, expand_idx=expand_idx, ep_recv_count=ep_recv_count,
-                      num_experts=num_experts)
-        return recv, scales, packed_recv_count, handle
+            counts = note["recv_per_expert"].cpu()          # the one host synchronisation (zbal_deepep.cpp:359, 379)
+            total = int(counts.sum().item())
+            rows = 1 if total == 0 else total               # zbal_deepep.cpp:360
+        qm = capi.QUANT_INT8 if use_quant else capi.NO_QUANT
+        recv_x, recv_x_scales, _, h = self.runtime.dispatch(x, topk_idx, topk_weights, num_tokens_per_expert, qm,
+                                                            recv_rows=rows, notified=note)
+        num_recv_tokens_per_expert_list: List[int] = []
+        if counts is not None:
+            run = 0
+            for c in counts.tolist():
+                run = run + int(c) if token_nums_type == 0 else int(c)
+                num_recv_tokens_per_expert_list.append(run)
+        handle = (is_token_in_rank, topk_idx, topk_weights, h["put_offset"], h["balance_matrix"])
+        return ((recv_x, recv_x_scales) if use_quant else recv_x, None, None, num_recv_tokens_per_expert_list, handle,
+                self._event(async_finish))
 
-    def low_latency_combine(self, x, topk_weights, handle):
-        """zbal_deepep.cpp:567-656."""
-        T, K = handle["expert_ids"].shape
-        H = x.shape[1]
-        out = self._empty((T, H), x.dtype)
-        capi.check("zbal_combine_low_latency", self.lib.zbal_combine_low_latency(
-            self._ti(x), self._ti(handle["expert_ids"]), self._ti(handle["expand_idx"], shape=(T, K)),
-            self._ti(handle["ep_recv_count"]), self._ti(topk_weights), self._ti(out), handle["num_experts"],
-            self.comm, capi.stream_ptr(), 0))
-        return out
+    def combine(self, x: torch.Tensor, handle: Tuple, topk_weights: Optional[torch.Tensor] = None,
+                bias: Union[torch.Tensor, Tuple[torch.Tensor, torch.Tensor]] = None, config: Optional[Config] = None,
+                previous_event: Optional[EventOverlap] = None, async_finish: bool = False,
+                allocate_on_comm_stream: bool = False, combine_send_cost_stats: Optional[torch.Tensor] = None
+                ) -> Tuple[torch.Tensor, Optional[torch.Tensor], EventOverlap]:
+        """zbal_buffer.py:350-411, zbal_deepep.cpp:395-452: out[t] = sum_k w[t, k] * x[row(t, k)] with the weights the
+        handle carries (those given to dispatch), as the reference. Returns (combined_x, None, event)."""
+        is_token_in_rank, topk_idx, topk_weights_ori, put_offset, balance_matrix = handle
+        if x.dim() != 2 or not x.is_contiguous():
+            raise ValueError("x dim not 2 or not contiguous")
+        if topk_weights_ori is None:
+            raise ValueError("topk_weights is empty")
+        if topk_weights_ori.dim() != 2 or topk_weights_ori.size(1) != topk_idx.size(1) or \
+                topk_weights_ori.dtype != torch.float32:
+            raise ValueError("topk_weights check failed")
+        self._wait(previous_event)
+        h = dict(put_offset=put_offset, balance_matrix=balance_matrix, expert_ids=topk_idx.to(torch.int32),
+                 send_token_idx=self.runtime.send_token_idx, num_experts=put_offset.size(1))
+        out = self.runtime.combine(x, h, topk_weights_ori)
+        return out, None, self._event(async_finish)
 
-    # -- fused MoE ------------------------------------------------------------------------------
-    def prepack_weight(self, w, int4=False):
-        """[E,K,N] one byte per element -> the library's pre-packed layout (the reference's format cast); shape stays [E,N,K]."""
-        E, K, N = w.shape
-        if int4:
-            dst = self._empty((E, N, K // 2), torch.uint8)
-            capi.check("zbal_moe_weight_prepack", self.lib.zbal_moe_weight_prepack(
-                self._ti(w), self._ti(dst, dtype=capi.DT_INT4X2), self.comm, capi.stream_ptr(), 0))
-        else:
-            dst = self._empty((E, N, K), w.dtype)
-            capi.check("zbal_moe_weight_prepack", self.lib.zbal_moe_weight_prepack(
-                self._ti(w), self._ti(dst), self.comm, capi.stream_ptr(), 0))
-        return dst
+    # ---- low-latency mode -----------------------------------------------------------------------------
+    def clean_low_latency_buffer(self, num_max_dispatch_tokens_per_rank: int, hidden: int, num_experts: int) -> None:
+        """zbal_buffer.py:413-430: nothing to clean (no flags live between calls)."""
+        return None
 
-    def fused_workspace_bytes(self, tokens, hidden, topk, num_experts, gmm1_h_len, quant_mode, share_gmm1_h_len=0):
-        n = self.lib.zbal_fused_deep_moe_workspace_size(tokens, hidden, topk, num_experts, gmm1_h_len, share_gmm1_h_len,
-                                                        quant_mode)
-        if n == 0:
-            raise ValueError("invalid fused MoE shape")
-        return int(n)
+    def low_latency_dispatch(self, x: torch.Tensor, topk_idx: torch.Tensor, num_max_dispatch_tokens_per_rank: int,
+                             num_experts: int, cumulative_local_expert_recv_stats: Optional[torch.Tensor] = None,
+                             use_fp8: bool = True, round_scale: bool = False, use_ue8m0: bool = False,
+                             async_finish: bool = False, return_recv_hook: bool = False
+                             ) -> Tuple[Union[Tuple[torch.Tensor, torch.Tensor], torch.Tensor], torch.Tensor, Tuple,
+                                        EventOverlap, Callable]:
+        """zbal_buffer.py:432-534, zbal_deepep.cpp:454-565. `use_fp8` means int8 rows with one fp32 scale per row, as
+        in the reference (zbal_deepep.cpp:514, 525). Rows are packed expert-major; packed_recv_count [experts] int64
+        holds counts (MOE_EXPERT_TOKEN_NUMS_TYPE=1, default) or their running sum (0). An empty batch is padded to
+        one token of ones that picks experts 0..topk-1, as the reference does.
+        Returns (recv_x or (recv_x, scales), packed_recv_count, handle, event, hook)."""
+        self._pad = None
+        new_x, new_idx = x, topk_idx
+        if topk_idx.size(0) < PADDING_SIZE:
+            pad = PADDING_SIZE - topk_idx.size(0)
+            K = topk_idx.size(1)
+            xs = [x] if topk_idx.size(0) != 0 else []
+            ts = [topk_idx] if topk_idx.size(0) != 0 else []
+            for _ in range(pad):
+                xs.append(torch.ones((1, x.size(1)), dtype=x.dtype, device=x.device))
+                ts.append(torch.arange(0, K, dtype=topk_idx.dtype, device=topk_idx.device).reshape(1, K))
+            new_x, new_idx = torch.cat(xs, 0), torch.cat(ts, 0)
+            self._pad = dict(count=pad, ori_x=x.clone(), topk_idx=new_idx)
+        recv, scales, packed_recv_count, h = self.runtime.low_latency_dispatch(
+            new_x, new_idx, num_max_dispatch_tokens_per_rank, num_experts, use_fp8=use_fp8)
+        handle = (h["expand_idx"], h["ep_recv_count"], num_max_dispatch_tokens_per_rank, x.size(1), num_experts,
+                  packed_recv_count)
+        kept = (x, topk_idx, recv, scales, packed_recv_count, h["expand_idx"], h["ep_recv_count"],
+                cumulative_local_expert_recv_stats)
+        return ((recv, scales) if use_fp8 else recv, packed_recv_count, handle,
+                self._event(async_finish, kept if async_finish else None), (lambda: None))
 
-    def fused_deep_moe(self, x, topk_idx, gmm1_permuted_weight, gmm1_permuted_weight_scale, gmm2_weight,
-                       gmm2_weight_scale, topk_weights, num_experts, quant_mode=0, expert_smooth_scales=None,
-                       share_gmm1_weight=None, share_gmm1_scale=None, share_gmm2_weight=None, share_gmm2_scale=None,
-                       share_smooth_scales=None, x_active_mask=None, workspace=None, out=None, is_tensor_list=False,
-                       share_out=None):
-        """zbal_deepep.cpp:658-802. Weights are pre-packed (prepack_weight; shared-expert weights as [1,N,K]).
-        Returns (output, share_output, expert_token_nums) like the reference; share_output is None without a shared
-        expert. x_active_mask [T] bool: only the first sum(mask) tokens are routed; the other rows of `out` keep
-        their contents. is_tensor_list: the four routed-expert operands are sequences of per-expert tensors (each
-        pre-packed on its own, [1,N,K] or [N,K]); the library receives one device table of addresses per operand."""
-        T, H = x.shape
-        K = topk_idx.shape[1]
-        n1 = gmm1_permuted_weight[0].shape[-2] if is_tensor_list else gmm1_permuted_weight.shape[1]
-        shared = share_gmm1_weight is not None
-        sn1 = share_gmm1_weight.shape[-2] if shared else 0
-        expert_ids = topk_idx if topk_idx.dtype == torch.int32 else topk_idx.to(torch.int32)
-        if workspace is None:
-            workspace = self._empty((self.fused_workspace_bytes(T, H, K, num_experts, n1, quant_mode, sn1),), torch.uint8)
-        if out is None:
-            out = self._empty((T, H), x.dtype)
-        if shared and share_out is None:
-            share_out = self._empty((T, H), x.dtype)
-        if not shared:
-            share_out = None
-        token_nums = self._empty((num_experts,), torch.int64)
-        wdt = {0: None, 1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[quant_mode]
-        null = ctypes.byref(capi.TensorInfo())
+    def low_latency_combine(self, x: torch.Tensor, topk_idx: torch.Tensor, topk_weights: torch.Tensor, handle: tuple,
+                            zero_copy: bool = False, async_finish: bool = False, return_recv_hook: bool = False,
+                            out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, EventOverlap, Callable]:
+        """zbal_buffer.py:536-609, zbal_deepep.cpp:567-656. x: the packed expert outputs, bf16.
+        Returns (combined_x, event, hook)."""
+        src_info, layout_range, num_max_dispatch_tokens_per_rank, hidden, num_experts, packed_recv_count = handle
+        if x.dim() != 2 or not x.is_contiguous() or x.dtype != torch.bfloat16:
+            raise ValueError("LL combine x check failed")
+        new_idx, new_scales = topk_idx, topk_weights
+        pad = self._pad
+        if pad is not None:
+            blocks = [topk_weights] if pad["count"] != PADDING_SIZE else []
+            blocks += [torch.zeros((1, topk_weights.size(1)), dtype=topk_weights.dtype, device=topk_weights.device)
+                       for _ in range(pad["count"])]
+            new_idx, new_scales = pad["topk_idx"], torch.cat(blocks, 0)
+        h = dict(expert_ids=new_idx.to(torch.int32), expand_idx=src_info, ep_recv_count=layout_range,
+                 num_experts=num_experts)
+        combined = self.runtime.low_latency_combine(x, new_scales, h)
+        if pad is not None:
+            combined = pad["ori_x"] if pad["count"] == PADDING_SIZE else combined[:PADDING_SIZE - pad["count"]]
+            self._pad = None
+        if out is not None:
+            out.copy_(combined)
+            combined = out
+        kept = (x, topk_idx, topk_weights, src_info, layout_range, combined)
+        return combined, self._event(async_finish, kept if async_finish else None), (lambda: None)
+
+    # ---- fused MoE --------------------------------------------------------------------------------------
+    def prepack_weight(self, w: torch.Tensor, int4: bool = False) -> torch.Tensor:
+        """[experts, K, N] one byte per element -> the library's pre-packed layout (this build's counterpart of the
+        reference's NZ format cast). The result is marked, so fused_deep_moe passes it through."""
+        p = self.runtime.prepack_weight(w, int4=int4)
+        p.zbal_prepacked = True
+        return p
+
+    def _packed_weight(self, w: torch.Tensor, int4: bool) -> torch.Tensor:
+        if getattr(w, "zbal_prepacked", False):
+            return w
+        key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
+        hit = self._packed.get(key)
+        if hit is None:
+            if len(self._packed) >= 16:
+                self._packed.clear()
+            w3 = w if w.dim() == 3 else w.unsqueeze(0)
+            hit = self.prepack_weight(w3.contiguous(), int4=int4)
+            self._packed[key] = hit
+        return hit
+
+    def topk_route(self, logits: torch.Tensor, num_topk: int, idx_dtype=torch.int64):
+        """Extension: softmax + top-k router; returns (topk_idx, topk_weights)."""
+        return self.runtime.topk_route(logits, num_topk, idx_dtype)
+
+    def fused_deep_moe(self, x: torch.Tensor, topk_idx: torch.Tensor, gmm1_permuted_weight: torch.Tensor,
+                       gmm1_permuted_weight_scale: torch.Tensor, gmm2_weight: torch.Tensor,
+                       gmm2_weight_scale: torch.Tensor, topk_weights: torch.Tensor, num_experts: int,
+                       shared_expert_num: int = 0, shared_expert_rank_num: int = 0, quant_mode: int = 0,
+                       num_max_dispatch_tokens_per_rank: int = 0, is_tensor_list: bool = False,
+                       expert_smooth_scales: Optional[torch.Tensor] = None,
+                       share_gmm1_weight: Optional[torch.Tensor] = None,
+                       share_gmm1_scale: Optional[torch.Tensor] = None,
+                       share_gmm2_weight: Optional[torch.Tensor] = None,
+                       share_gmm2_scale: Optional[torch.Tensor] = None,
+                       share_smooth_scales: Optional[torch.Tensor] = None,
+                       x_active_mask: Optional[torch.Tensor] = None, share_gmm1_h_len: int = 0, fuse_mode: int = 0
+                       ) -> Tuple[torch.Tensor, torch.Tensor]:
+        """zbal_buffer.py:611-710, zbal_deepep.cpp:658-802: quantise -> permute -> GMM1 -> SwiGLU -> requantise -> GMM2
+        -> weighted combine in one call. Weights [experts, hidden, gmm1_h_len] / [experts, gmm1_h_len/2, hidden], one
+        byte per element (quant_mode 0 or 1: int8 with per-channel scales, the reference's only mode; 2 = e4m3 with
+        128x128 block scales; 3 = int4 values in int8 storage with fp16 group scales), or tensor lists of per-expert
+        tensors with is_tensor_list. The shared expert's output is kept in `last_share_output`.
+        Returns (output [tokens, hidden], expert_token_nums [experts] int64)."""
+        has_share = share_gmm1_weight is not None and share_gmm1_weight.numel() > 0
+        if has_share and share_gmm1_h_len <= 0:
+            print("[ZBAL WARNING] share_gmm1_weight provided but share_gmm1_h_len is not set (or <=0). "
+                  "Please pass share_gmm1_h_len with the correct value to avoid kernel errors.")
+        int4 = quant_mode == 3
         if is_tensor_list:
-            def wti(t, **kw):
-                return self._list_ti(t, num_experts, **kw)
+            w1 = [self._packed_weight(t, int4) for t in gmm1_permuted_weight]
+            w2 = [self._packed_weight(t, int4) for t in gmm2_weight]
         else:
-            wti = self._ti
-        capi.check("zbal_fused_deep_moe", self.lib.zbal_fused_deep_moe(
-            self._ti(x), self._ti(expert_ids),
-            wti(gmm1_permuted_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED),
-            wti(gmm1_permuted_weight_scale),
-            wti(gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED), wti(gmm2_weight_scale),
-            self._ti(topk_weights), self._ti(expert_smooth_scales) if expert_smooth_scales is not None else null,
-            self._ti(share_gmm1_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED) if shared else null,
-            self._ti(share_gmm1_scale) if shared else null,
-            self._ti(share_gmm2_weight, dtype=wdt, weight_format=capi.WEIGHT_FORMAT_PREPACKED) if shared else null,
-            self._ti(share_gmm2_scale) if shared else null,
-            self._ti(share_smooth_scales) if share_smooth_scales is not None else null,
-            self._ti(x_active_mask.view(torch.uint8)) if x_active_mask is not None else null,
-            self._ti(out), self._ti(share_out) if shared else null, self._ti(token_nums), self._ti(workspace),
-            num_experts, quant_mode, 0, n1, sn1, int(is_tensor_list), self.comm, capi.stream_ptr(), 0))
-        return out, share_out, token_nums
+            w1, w2 = self._packed_weight(gmm1_permuted_weight, int4), self._packed_weight(gmm2_weight, int4)
+        sw1 = self._packed_weight(share_gmm1_weight, int4) if has_share else None
+        sw2 = self._packed_weight(share_gmm2_weight, int4) if has_share else None
+        out, share_out, nums = self.runtime.fused_deep_moe(
+            x, topk_idx.int(), w1, gmm1_permuted_weight_scale, w2, gmm2_weight_scale, topk_weights, num_experts,
+            quant_mode=quant_mode, expert_smooth_scales=expert_smooth_scales, share_gmm1_weight=sw1,
+            share_gmm1_scale=share_gmm1_scale if has_share else None, share_gmm2_weight=sw2,
+            share_gmm2_scale=share_gmm2_scale if has_share else None, share_smooth_scales=share_smooth_scales,
+            x_active_mask=x_active_mask, is_tensor_list=is_tensor_list)
+        self.last_share_output = share_out
+        return out, nums

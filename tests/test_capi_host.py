@@ -222,3 +222,56 @@ def test_kernel_seam_types_and_exports():
                      "ZBALOpDispatchNormal", "ZBALOpCombineNormal", "ZBALOpDispatchLowLatency", "ZBALOpCombineLowLatency",
                      "ZBALOpFusedDeepMoe"}
     assert set(capi.CXX_SIGNATURES) <= names
+
+
+def test_deepep_buffer_signatures_follow_the_reference():
+    """Parameter names, order and defaults of the DeepEP-compatible Buffer, as the reference's Python face declares
+    them (app/zbal/src/python/zbal/zbal_buffer.py:28-37, 168-175, 216-232, 350-360, 432-443, 536-545, 611-634)."""
+    import inspect
+    from memfabric_hybrid_amd.buffer import Buffer, Config, EventOverlap
+
+    def sig(fn):
+        return [(n, p.default if p.default is not inspect.Parameter.empty else "<required>")
+                for n, p in inspect.signature(fn).parameters.items() if n != "self"]
+
+    assert sig(Buffer.__init__)[:7] == [
+        ("group", None), ("num_nvl_bytes", 0), ("num_rdma_bytes", 0), ("low_latency_mode", False),
+        ("num_qps_per_rank", 12), ("allow_nvlink_for_low_latency_mode", True), ("allow_mnnvl", False)]
+    assert sig(Buffer.get_dispatch_layout) == [
+        ("topk_idx", "<required>"), ("num_experts", "<required>"), ("previous_event", None), ("async_finish", False),
+        ("allocate_on_comm_stream", False)]
+    assert sig(Buffer.dispatch) == [
+        ("x", "<required>"), ("handle", None), ("num_tokens_per_rank", None), ("num_tokens_per_rdma_rank", None),
+        ("is_token_in_rank", None), ("num_tokens_per_expert", None), ("topk_idx", None), ("topk_weights", None),
+        ("expert_alignment", 1), ("num_worst_tokens", 0), ("config", None), ("previous_event", None),
+        ("async_finish", False), ("allocate_on_comm_stream", False), ("dispatch_wait_recv_cost_stats", None)]
+    assert sig(Buffer.combine) == [
+        ("x", "<required>"), ("handle", "<required>"), ("topk_weights", None), ("bias", None), ("config", None),
+        ("previous_event", None), ("async_finish", False), ("allocate_on_comm_stream", False),
+        ("combine_send_cost_stats", None)]
+    assert sig(Buffer.low_latency_dispatch) == [
+        ("x", "<required>"), ("topk_idx", "<required>"), ("num_max_dispatch_tokens_per_rank", "<required>"),
+        ("num_experts", "<required>"), ("cumulative_local_expert_recv_stats", None), ("use_fp8", True),
+        ("round_scale", False), ("use_ue8m0", False), ("async_finish", False), ("return_recv_hook", False)]
+    assert sig(Buffer.low_latency_combine) == [
+        ("x", "<required>"), ("topk_idx", "<required>"), ("topk_weights", "<required>"), ("handle", "<required>"),
+        ("zero_copy", False), ("async_finish", False), ("return_recv_hook", False), ("out", None)]
+    assert sig(Buffer.fused_deep_moe) == [
+        ("x", "<required>"), ("topk_idx", "<required>"), ("gmm1_permuted_weight", "<required>"),
+        ("gmm1_permuted_weight_scale", "<required>"), ("gmm2_weight", "<required>"), ("gmm2_weight_scale", "<required>"),
+        ("topk_weights", "<required>"), ("num_experts", "<required>"), ("shared_expert_num", 0),
+        ("shared_expert_rank_num", 0), ("quant_mode", 0), ("num_max_dispatch_tokens_per_rank", 0),
+        ("is_tensor_list", False), ("expert_smooth_scales", None), ("share_gmm1_weight", None),
+        ("share_gmm1_scale", None), ("share_gmm2_weight", None), ("share_gmm2_scale", None),
+        ("share_smooth_scales", None), ("x_active_mask", None), ("share_gmm1_h_len", 0), ("fuse_mode", 0)]
+    assert sig(Buffer.clean_low_latency_buffer) == [
+        ("num_max_dispatch_tokens_per_rank", "<required>"), ("hidden", "<required>"), ("num_experts", "<required>")]
+    c = Buffer.get_dispatch_config(8)
+    assert isinstance(c, Config) and (c.num_sms, c.num_max_nvl_chunked_send_tokens, c.num_max_nvl_chunked_recv_tokens,
+                                      c.num_max_rdma_chunked_send_tokens, c.num_max_rdma_chunked_recv_tokens) == \
+        (Buffer.num_sms, 6, 256, 6, 128)
+    c = Buffer.get_combine_config(32)
+    assert (c.num_max_nvl_chunked_send_tokens, c.num_max_nvl_chunked_recv_tokens) == (1, 288)
+    assert c.get_nvl_buffer_size_hint(14336, 8) == 14336 and c.get_rdma_buffer_size_hint(14336, 8) == 14336
+    assert Buffer.get_low_latency_rdma_size_hint(128, 7168, 8, 256) == 128
+    assert EventOverlap().current_stream_wait() is None

@@ -32,7 +32,7 @@ def test_oracle_reproduces_fixture():
 def test_gpu_reproduces_fixture():
     import torch
     from memfabric_hybrid_amd import capi
-    from memfabric_hybrid_amd.buffer import Buffer
+    from memfabric_hybrid_amd.operators import OperatorBuffer as Buffer
     from oracle import oracle as zo
     from zbal_testlib import dev, host, max_rel_err
     c = mk.cfg1_inputs()

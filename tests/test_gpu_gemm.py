@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from memfabric_hybrid_amd import capi
-from memfabric_hybrid_amd.buffer import Buffer
+from memfabric_hybrid_amd.operators import OperatorBuffer as Buffer
 from oracle import oracle as zo
 from zbal_testlib import FP8_GEMM_ELEM_TOL, assert_fp8_close, bf16_normal, calc_diff, dev, distinct_topk, host, max_rel_err, rng
 

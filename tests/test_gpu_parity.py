@@ -8,7 +8,7 @@ import pytest
 import torch
 
 from memfabric_hybrid_amd import capi
-from memfabric_hybrid_amd.buffer import Buffer
+from memfabric_hybrid_amd.operators import OperatorBuffer as Buffer
 from oracle import oracle as zo
 from zbal_testlib import bf16_normal, calc_diff, dev, distinct_topk, host, max_rel_err, rng
 
@@ -270,7 +270,7 @@ def test_reduce_full_size_sampled_windows(buf):
 
 def test_reduce_scatter_and_all_reduce_over_peer_windows(buf):
     """cfg4 shape in miniature: 8 'ranks' as local windows, this rank reduces its slice of every peer's buffer."""
-    from memfabric_hybrid_amd.buffer import create_group, destroy_group
+    from memfabric_hybrid_amd.operators import create_group, destroy_group
     lib = buf.lib
     R, me, n = 8, 5, 6 * 2 ** 12
     comm = create_group("rs8", R, me)
@@ -313,7 +313,7 @@ def test_device_trace_ring_and_trace_viewer_dump(buf, tmp_path, monkeypatch):
     is destroyed. Results must not change."""
     import glob
     import json
-    from memfabric_hybrid_amd.buffer import create_group, destroy_group
+    from memfabric_hybrid_amd.operators import create_group, destroy_group
     lib = buf.lib
     monkeypatch.setenv("ZBAL_PROF_ENABLE", "1")
     monkeypatch.setenv("ZBAL_PROF_DIR", str(tmp_path))

@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from memfabric_hybrid_amd import capi
-from memfabric_hybrid_amd.buffer import Buffer, create_group, destroy_group
+from memfabric_hybrid_amd.operators import OperatorBuffer as Buffer, create_group, destroy_group
 from oracle import oracle as zo
 from zbal_testlib import bf16_normal, host, rng
 
