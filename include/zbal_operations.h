@@ -66,6 +66,26 @@ int32_t zbal_all_reduce(const void *send_buff, void *recv_buff, void *buffer, si
 int32_t zbal_reduce_scatter(const void *sendBuff, void *recvBuff, size_t recv_count, zbal_datatype_t dataType,
                             zbal_reduce_op_t op, zbal_comm_t comm, aclrtStream stream);
 
+/*
+ * reference zbal_operations.h:111-209. The data-movement collectives need a transport between devices, which
+ * is not part of this build: they are exported so that a client of the reference links unchanged, validate
+ * nothing, set the last-error text and return Z_INVALID_PARAM.
+ */
+int32_t zbal_all_gather(const void *sendBuff, void *recvBuff, size_t send_count, zbal_datatype_t dataType,
+                        zbal_comm_t comm, aclrtStream stream);
+int32_t zbal_all_to_all_v(const void *sendBuff, void *recvBuff, void *sendCumSum, void *recvSplitCounts, void *elements,
+                          zbal_datatype_t dataType, zbal_comm_t comm, aclrtStream stream);
+int32_t zbal_broadcast(const void *buf, uint64_t data_count, zbal_datatype_t dataType, uint16_t root, zbal_comm_t comm,
+                       aclrtStream stream);
+int32_t zbal_scatter(const void *sendBuff, void *recvBuff, uint64_t data_count, zbal_datatype_t dataType, uint16_t root,
+                     zbal_comm_t comm, aclrtStream stream);
+int32_t zbal_gather(const void *sendBuff, void *recvBuff, uint64_t data_count, zbal_datatype_t dataType, uint16_t root,
+                    zbal_comm_t comm, aclrtStream stream);
+int32_t zbal_barrier(zbal_comm_t comm, aclrtStream stream);
+int32_t zbal_send(const void *sendBuff, zbal_datatype_t dataType, uint32_t peer, zbal_comm_t comm, aclrtStream stream);
+int32_t zbal_recv(const void *recvBuff, size_t recvCount, zbal_datatype_t dataType, uint32_t peer, zbal_comm_t comm,
+                  aclrtStream stream);
+
 /* reference zbal_operations.h:227-231 */
 int32_t zbal_dispatch_normal_notify(const zbal_tensor_info_t *sendTokensPerExpert, int64_t sendCount, int64_t topKNum,
                                     const zbal_tensor_info_t *recvBuff, const zbal_tensor_info_t *totalRecvTokens,

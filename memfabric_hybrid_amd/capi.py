@@ -105,6 +105,15 @@ SIGNATURES = {
     "zbal_comm_dump_profiling_trace": (_i32, [_vp]),
     "zbal_all_reduce": (_i32, [_vp, _vp, _vp, ctypes.c_size_t, _i32, _i32, _vp, _vp]),
     "zbal_reduce_scatter": (_i32, [_vp, _vp, ctypes.c_size_t, _i32, _i32, _vp, _vp]),
+    # exported for link compatibility; every one of them refuses (no transport between devices in this build)
+    "zbal_all_gather": (_i32, [_vp, _vp, ctypes.c_size_t, _i32, _vp, _vp]),
+    "zbal_all_to_all_v": (_i32, [_vp, _vp, _vp, _vp, _vp, _i32, _vp, _vp]),
+    "zbal_broadcast": (_i32, [_vp, ctypes.c_uint64, _i32, _u16, _vp, _vp]),
+    "zbal_scatter": (_i32, [_vp, _vp, ctypes.c_uint64, _i32, _u16, _vp, _vp]),
+    "zbal_gather": (_i32, [_vp, _vp, ctypes.c_uint64, _i32, _u16, _vp, _vp]),
+    "zbal_barrier": (_i32, [_vp, _vp]),
+    "zbal_send": (_i32, [_vp, _i32, _u32, _vp, _vp]),
+    "zbal_recv": (_i32, [_vp, ctypes.c_size_t, _i32, _u32, _vp, _vp]),
     "zbal_dispatch_normal_notify": (_i32, [_TI, _i64, _i64, _TI, _TI, _TI, _TI, _TI, _vp, _vp, _i64]),
     "zbal_dispatch_normal_layout": (_i32, [_TI, _i64, _i64, _i64, _TI, _TI, _TI, _TI, _vp, _vp, _i64]),
     "zbal_dispatch_normal": (_i32, [_TI, _TI, _TI, _TI, _TI, _i64, _i32, _TI, _TI, _vp, _vp, _i64]),

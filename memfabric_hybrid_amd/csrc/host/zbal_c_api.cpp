@@ -168,6 +168,23 @@ ZBAL_API int32_t zbal_reduce_scatter(const void *sendBuff, void *recvBuff, size_
     return c->ReduceScatter(sendBuff, recvBuff, recv_count, dataType, op, stream);
 }
 
+/* ---- data-movement collectives: exported for link compatibility, refused (no transport between devices here) ---- */
+
+static int32_t NoTransport(const char *op)
+{
+    ZBAL_LOG_AND_SET_LAST_ERROR(op << " failed as this build has no transport between devices");
+    return Z_INVALID_PARAM;
+}
+
+ZBAL_API int32_t zbal_all_gather(const void *, void *, size_t, zbal_datatype_t, zbal_comm_t, aclrtStream) { return NoTransport("AllGather"); }
+ZBAL_API int32_t zbal_all_to_all_v(const void *, void *, void *, void *, void *, zbal_datatype_t, zbal_comm_t, aclrtStream) { return NoTransport("AllToAllV"); }
+ZBAL_API int32_t zbal_broadcast(const void *, uint64_t, zbal_datatype_t, uint16_t, zbal_comm_t, aclrtStream) { return NoTransport("Broadcast"); }
+ZBAL_API int32_t zbal_scatter(const void *, void *, uint64_t, zbal_datatype_t, uint16_t, zbal_comm_t, aclrtStream) { return NoTransport("Scatter"); }
+ZBAL_API int32_t zbal_gather(const void *, void *, uint64_t, zbal_datatype_t, uint16_t, zbal_comm_t, aclrtStream) { return NoTransport("Gather"); }
+ZBAL_API int32_t zbal_barrier(zbal_comm_t, aclrtStream) { return NoTransport("Barrier"); }
+ZBAL_API int32_t zbal_send(const void *, zbal_datatype_t, uint32_t, zbal_comm_t, aclrtStream) { return NoTransport("Send"); }
+ZBAL_API int32_t zbal_recv(const void *, size_t, zbal_datatype_t, uint32_t, zbal_comm_t, aclrtStream) { return NoTransport("Recv"); }
+
 /* ---- MoE operators: reference zbal_operations.cpp:258-457 ----------------------- */
 
 ZBAL_API int32_t zbal_dispatch_normal_notify(const zbal_tensor_info_t *sendTokensPerExpert, int64_t sendCount,

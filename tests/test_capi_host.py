@@ -275,3 +275,11 @@ def test_deepep_buffer_signatures_follow_the_reference():
     assert c.get_nvl_buffer_size_hint(14336, 8) == 14336 and c.get_rdma_buffer_size_hint(14336, 8) == 14336
     assert Buffer.get_low_latency_rdma_size_hint(128, 7168, 8, 256) == 128
     assert EventOverlap().current_stream_wait() is None
+
+
+def test_data_movement_collectives_link_and_refuse(lib):
+    """A client of the reference that names these still links; each call says why it cannot run here."""
+    assert lib.zbal_barrier(None, None) == capi.Z_INVALID_PARAM
+    assert "no transport" in capi.last_error()
+    assert lib.zbal_all_gather(None, None, 0, 0, None, None) == capi.Z_INVALID_PARAM
+    assert lib.zbal_send(None, 0, 0, None, None) == capi.Z_INVALID_PARAM
