@@ -380,6 +380,40 @@ notify_ranks_kernel(CountsOfRanks counts, int ranks, int me, int experts, int to
  * One wave per token; lane l holds logits l, l + 64, ... (PER_LANE of them: the launcher picks the smallest
  * instantiation that covers `experts`, the arithmetic and its order are the same in all of them).
  */
+/*
+ * Up to 64 experts: one logit per lane, and no serial rounds of wave arg-max. A lane's pick position is its rank:
+ * the number of logits that are larger, or equal with a lower index (the order K rounds of arg-max with ties to
+ * the lower index produce). Ranks come from one pass over the experts with the logit of expert m read from lane m
+ * as a scalar; maximum and sums run on the DPP path. Same formulas as the general kernel below
+ * (p = exp(l - max) / sum; weight = p / sum of the picked p), sums taken in a different order.
+ */
+__global__ void __launch_bounds__(256)
+topk_route_small_kernel(const float *__restrict__ logits, int tokens, int experts, int topk, void *__restrict__ topk_idx,
+                        int idx_is_i64, float *__restrict__ topk_w)
+{
+    const int lane = threadIdx.x & 63;
+    const int t = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (t >= tokens) return; /* whole waves leave together */
+    const bool mine = lane < experts;
+    const float v = mine ? logits[(int64_t)t * experts + lane] : -__builtin_inff();
+    const float mx = zb_wave_reduce_dpp<true>(v);
+    const float ex = mine ? zb_expf(v - mx) : 0.0f;
+    const float sum = zb_wave_reduce_dpp<false>(ex);
+    int rank = 0;
+    for (int m = 0; m < experts; ++m) {
+        const float s = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), m));
+        rank += (s > v || (s == v && m < lane)) ? 1 : 0;
+    }
+    const bool picked = mine && rank < topk;
+    const float p = ex / sum;
+    const float wsum = zb_wave_reduce_dpp<false>(picked ? p : 0.0f);
+    if (picked) {
+        if (idx_is_i64) static_cast<int64_t *>(topk_idx)[(int64_t)t * topk + rank] = lane;
+        else static_cast<int32_t *>(topk_idx)[(int64_t)t * topk + rank] = lane;
+        topk_w[(int64_t)t * topk + rank] = p / wsum;
+    }
+}
+
 template <int PER_LANE>
 __global__ void __launch_bounds__(256)
 topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int topk, void *__restrict__ topk_idx,
@@ -532,7 +566,7 @@ extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64
     const int64_t blocks = (tokens + wpb - 1) / wpb;
     const dim3 grid((unsigned)blocks), block(wpb * 64);
     hipStream_t st = (hipStream_t)stream;
-    if (experts <= 64) topk_route_kernel<1><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
+    if (experts <= 64) topk_route_small_kernel<<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     else if (experts <= 256) topk_route_kernel<4><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     else topk_route_kernel<ZB_MAX_EXPERTS / 64><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     return zbalhip_check_launch();

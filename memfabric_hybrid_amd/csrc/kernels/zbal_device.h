@@ -11,6 +11,7 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 
 #define ZBALHIP_OK 0
 #define ZBALHIP_INVALID (-2)
@@ -147,6 +148,28 @@ __device__ __forceinline__ float zb_wave_max(float v)
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, ZBAL_WAVE));
     return v;
+}
+
+/*
+ * Wave-wide reductions on the data-parallel-primitive path (no LDS round trips: six dependent vector instructions
+ * instead of six ds_bpermute latencies). Lanes swap within quads, mirror within 8 and 16, then rows 1 and 3 take
+ * the totals of rows 0 and 2 and the upper half takes lane 31's; lane 63 ends with the result, which is broadcast.
+ */
+template <bool IS_MAX> __device__ __forceinline__ float zb_wave_reduce_dpp(float x)
+{
+    const int ident = IS_MAX ? (int)0xff800000u : 0;       /* -inf or +0 for the lanes a step does not write */
+    auto step = [&](auto ctrl_tag, auto mask_tag) __attribute__((always_inline)) {
+        constexpr int CTRL = decltype(ctrl_tag)::value, MASK = decltype(mask_tag)::value;
+        const float o = __int_as_float(__builtin_amdgcn_update_dpp(ident, __float_as_int(x), CTRL, MASK, 0xf, false));
+        x = IS_MAX ? fmaxf(x, o) : x + o;
+    };
+    step(std::integral_constant<int, 0xB1>{}, std::integral_constant<int, 0xf>{});     /* quad_perm [1,0,3,2] */
+    step(std::integral_constant<int, 0x4E>{}, std::integral_constant<int, 0xf>{});     /* quad_perm [2,3,0,1] */
+    step(std::integral_constant<int, 0x141>{}, std::integral_constant<int, 0xf>{});    /* row_half_mirror */
+    step(std::integral_constant<int, 0x140>{}, std::integral_constant<int, 0xf>{});    /* row_mirror */
+    step(std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{});    /* row_bcast:15 into rows 1 and 3 */
+    step(std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xc>{});    /* row_bcast:31 into rows 2 and 3 */
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), 63));
 }
 
 /* max over groups of 2^LOG2 consecutive lanes */
