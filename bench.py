@@ -213,9 +213,9 @@ def bench_moe(args, torch, np, capi, buf, workload):
     # ---- the same stages one by one through the inner kernel ABI, with events between them -----------------
     off = {k: int(v) for k, v in plan_workspace(lib, T, H, K, E, N1, mode).items()}
     base = ws.data_ptr()
-    q1, xs, eidx, row_off, scratch, q2, sc2, y = (base + off[k] for k in
-                                                  ("q1", "xs", "expand_idx", "row_off", "layout_scratch", "q2", "scale2", "y"))
+    q1, xs, eidx, row_off, q2, sc2, y = (base + off[k] for k in ("q1", "xs", "expand_idx", "row_off", "q2", "scale2", "y"))
     sgl = base + off["sgl"] if mode != 2 else None
+    rowmax = sgl + rows * I * 4 if sgl else None      # int modes: row maxima behind the fp32 SwiGLU values; the permute launch clears them
     names = ["route", "permute_quant", "gmm1_swiglu_quant", "gmm2_dequant", "combine"]
     s2dt = {1: capi.DT_BF16, 2: capi.DT_FP32, 3: capi.DT_FP16}[mode]
 
@@ -227,9 +227,10 @@ def bench_moe(args, torch, np, capi, buf, workload):
         evs[1].record()
         capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, None, T, H, K, E,
                                                               2 if mode == 2 else 1, q1, xs, eidx, nums.data_ptr(), row_off,
-                                                              scratch, 50, st))
+                                                              rowmax, rows if rowmax else 0, st))
         evs[2].record()
-        capi.check("gmm1", lib.zbalhip_gmm1_swiglu_quant(q1, xs, w1.data_ptr(), s1.data_ptr(), row_off, E, rows, H, N1, mode,
+        capi.check("gmm1", lib.zbalhip_gmm1_swiglu_quant(q1, xs, w1.data_ptr(), s1.data_ptr(), row_off, E, rows, H, N1,
+                                                         mode | (capi.ROWMAX_CLEARED if rowmax else 0),
                                                          q2, sc2, sgl, st))
         evs[3].record()
         capi.check("gmm2", lib.zbalhip_gmm2_dequant(q2, sc2, w2.data_ptr(), s2.data_ptr(), s2dt, row_off, E, rows, I,

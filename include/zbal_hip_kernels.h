@@ -205,8 +205,12 @@ ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int
  * 952-995, 1859-2058). mode 1: int8, s = 127/amax, optional smooth [E,H]
  * fp32 multiplied in first; mode 2: e4m3 1x128. Outputs q1 [rows,H], xs
  * ([rows] or [rows,H/128]), expand_idx [T,K], counts [E] i64 and the
- * exclusive row offsets row_off [E+1] i32. scratch / scratch_blocks as above
- * (not touched). active_mask (optional, one byte per token): only the first
+ * exclusive row offsets row_off [E+1] i32. The launch also sets clear_count
+ * 32-bit words at clear_words to zero (0 / null for none): the row maxima that
+ * the int modes' first GEMM accumulates into, so that it needs no fill launch
+ * of its own (ZBALHIP_ROWMAX_CLEARED). With at most 4096 picks (tokens x topk)
+ * the permute kernel works the layout out itself and the stage is one launch.
+ * active_mask (optional, one byte per token): only the first
  * sum(mask) tokens are routed, as in the reference's TokenActiveMaskCal
  * (…swiglu_quant_multistage_workspace.h:836-863); the picks of the others get
  * expand_idx = -1, which zbalhip_combine reads as "leave this token's output
@@ -216,7 +220,7 @@ ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, 
                                     const uint8_t *active_mask,
                                     int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int32_t mode,
                                     void *q1, float *xs, int32_t *expand_idx, int64_t *counts, int32_t *row_off,
-                                    int32_t *scratch, int32_t scratch_blocks, void *stream);
+                                    uint32_t *clear_words, int64_t clear_count, void *stream);
 
 /*
  * OR-ed into `mode` of the two grouped GEMMs: `w1`/`w2` and their scales are
@@ -226,6 +230,13 @@ ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, 
  * …swiglu_quant_multistage_workspace.h:669-673, 755-757, 1531-1558).
  */
 #define ZBALHIP_WEIGHTS_AS_LISTS 0x100
+/*
+ * OR-ed into `mode` of zbalhip_gmm1_swiglu_quant (int modes): the row maxima
+ * behind the SwiGLU values in sgl_ws (max_rows words at sgl_ws + max_rows *
+ * N1/2) are already zero - the permute launch cleared them - so the GEMM
+ * launches no fill kernel of its own.
+ */
+#define ZBALHIP_ROWMAX_CLEARED 0x200
 
 /*
  * Grouped GEMM 1 with dequant + SwiGLU + requant epilogue (AIC loop

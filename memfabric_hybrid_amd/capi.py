@@ -22,6 +22,7 @@ DT_UINT8, DT_UINT16, DT_UINT32, DT_FP8_E4M3, DT_INT4X2 = 9, 10, 11, 12, 13
 REDUCE_PROD, REDUCE_SUM, REDUCE_MAX, REDUCE_MIN = 0, 1, 2, 3
 # zbal_quant_mode_t
 NO_QUANT, QUANT_INT8, QUANT_FP8_B128, QUANT_W4A8_G128 = 0, 1, 2, 3
+ROWMAX_CLEARED = 0x200   # ZBALHIP_ROWMAX_CLEARED: OR-ed into the mode of zbalhip_gmm1_swiglu_quant
 # zbal_backend_t
 BACKEND_GPU, BACKEND_DUMMY = 0, 1
 WEIGHT_FORMAT_ND, WEIGHT_FORMAT_PREPACKED = 0, 1
@@ -142,7 +143,7 @@ SIGNATURES = {
     "zbalhip_weight_prepack": (_i32, [_vp, _i64, _i64, _i64, _i32, _vp, _vp]),
     "zbalhip_fill_i32": (_i32, [_vp, _i64, _i32, _vp]),
     "zbalhip_fused_permute_quant": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp,
-                                           _vp, _i32, _vp]),
+                                           _vp, _i64, _vp]),
     "zbalhip_gmm1_swiglu_quant": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "zbalhip_gmm2_dequant": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp, _vp]),
 }

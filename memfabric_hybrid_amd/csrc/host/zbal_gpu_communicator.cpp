@@ -629,7 +629,6 @@ public:
         float *xs = (float *)(base + ws.xs);
         int32_t *expandIdx = (int32_t *)(base + ws.expand_idx);
         int32_t *rowOff = (int32_t *)(base + ws.row_off);
-        int32_t *scratch = (int32_t *)(base + ws.layout_scratch);
         void *q2 = base + ws.q2;
         float *scale2 = (float *)(base + ws.scale2);
         float *sgl = mode == 2 ? nullptr : (float *)(base + ws.sgl);
@@ -637,11 +636,12 @@ public:
         const int qmode = mode == 2 ? 2 : 1;
         /* tensor lists: the four routed-expert descriptors point at device tables of one address per expert */
         const int32_t gemmMode = mode | (isTensorList ? ZBALHIP_WEIGHTS_AS_LISTS : 0);
+        /* int modes: the permute launch clears the row maxima the first GEMM accumulates into (no fill launch) */
+        const int32_t clearedFlag = sgl ? ZBALHIP_ROWMAX_CLEARED : 0;
         if (T == 0) { /* nothing routed: counts are zero */
             return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth,
                                                             nullptr, 0, H, K, E, qmode, q1, xs, expandIdx,
-                                                            (int64_t *)expertTokenNums->data, rowOff, scratch,
-                                                            ZBALHIP_LAYOUT_MAX_BLOCKS, stream));
+                                                            (int64_t *)expertTokenNums->data, rowOff, nullptr, 0, stream));
         }
         int32_t rc = 0;
         if (shared) {
@@ -657,21 +657,21 @@ public:
             if (rc != 0) return Launched(op, rc);
             /* with x_active_mask the shared expert, too, sees only the first sum(mask) tokens (TokenActiveMaskCal) */
             rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, activeMask, T, H, 1, 1, qmode, q1, xs, expandIdx,
-                                             shareCount, rowOff, scratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
+                                             shareCount, rowOff, sgl ? (uint32_t *)(sgl + T * SI) : nullptr, sgl ? T : 0, stream);
             if (rc != 0) return Launched(op, rc);
-            rc = zbalhip_gmm1_swiglu_quant(q1, xs, shareGmm1Weight->data, shareGmm1Scale->data, rowOff, 1, T, H, SN1, mode,
-                                           q2, scale2, sgl, stream);
+            rc = zbalhip_gmm1_swiglu_quant(q1, xs, shareGmm1Weight->data, shareGmm1Scale->data, rowOff, 1, T, H, SN1,
+                                           mode | clearedFlag, q2, scale2, sgl, stream);
             if (rc != 0) return Launched(op, rc);
             rc = zbalhip_gmm2_dequant(q2, scale2, shareGmm2Weight->data, shareGmm2Scale->data, shareWscale2Dt, rowOff, 1, T,
                                       SI, H, mode, x->dataType, shareOutput->data, stream);
             if (rc != 0) return Launched(op, rc);
         }
         rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, activeMask, T, H, K, E,
-                                         qmode, q1, xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff, scratch,
-                                         ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
+                                         qmode, q1, xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff,
+                                         sgl ? (uint32_t *)(sgl + rows * I) : nullptr, sgl ? rows : 0, stream);
         if (rc != 0) return Launched(op, rc);
-        rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1, gemmMode, q2,
-                                       scale2, sgl, stream);
+        rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1,
+                                       gemmMode | clearedFlag, q2, scale2, sgl, stream);
         if (rc != 0) return Launched(op, rc);
         rc = zbalhip_gmm2_dequant(q2, scale2, gmm2Weight->data, gmm2Scale->data, wscale2Dt, rowOff, E, rows, I, H, gemmMode,
                                   x->dataType, y, stream);

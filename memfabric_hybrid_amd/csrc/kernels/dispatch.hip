@@ -48,6 +48,98 @@ __device__ __forceinline__ int64_t pick_row(const int32_t *__restrict__ base, in
     return row < pr.rows_cap ? row : -1;
 }
 
+/*
+ * Small batches: the permute kernel works the layout out itself. With at most kInlineMaxPicks picks in all, every
+ * workgroup counts the whole index array (a few KiB that sit in L2) into an LDS histogram, scans it into the
+ * exclusive row offsets and counts the same-expert picks that precede each of its own token's picks: no layout
+ * launch in front of the permute, and no dependency between workgroups. Workgroup 0 also writes the layout's
+ * outputs (any of them may be null); every workgroup writes its token's expand_idx entries.
+ */
+constexpr int kInlineMaxPicks = 4096;
+constexpr int kInlineMaxTopk = 32;
+constexpr int kInlineMaxExperts = 1024;
+
+struct InlineLayout {
+    const uint8_t *active_mask;   /* optional: only the first sum(mask) tokens are routed */
+    int tokens, token_nums_type;
+    int32_t *expand_idx;          /* [T, K] */
+    int32_t *incl_i32;            /* [E] running sums */
+    int32_t *row_off;             /* [E + 1] exclusive offsets */
+    int64_t *counts_i64;          /* [E] */
+    int64_t *nums_typed;          /* [E] counts (type 1) or running sums (type 0) */
+};
+
+/* on return s_off[e] = rows before expert e, s_e[k] / s_rk[k] = expert and rank of pick k of token t (rank -1: not routed) */
+__device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, int t, int topk, int experts,
+                                              const InlineLayout &il, int32_t *s_off, int32_t *s_e, int32_t *s_rk, int32_t *s_tmp)
+{
+    const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6;
+    for (int e = tid; e < experts; e += nthr) s_off[e] = 0;
+    if (tid < topk) {
+        s_e[tid] = idx[(int64_t)t * topk + tid];
+        s_rk[tid] = 0;
+    }
+    if (tid == 0) s_tmp[0] = 0;
+    __syncthreads();
+    int active = il.tokens;
+    if (il.active_mask) {
+        int part = 0;
+        for (int tt = tid; tt < il.tokens; tt += nthr) part += il.active_mask[tt] != 0;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if (lane == 0 && part) atomicAdd(&s_tmp[0], part);
+        __syncthreads();
+        active = s_tmp[0];
+    }
+    const int n = active * topk, mine0 = t * topk;
+    for (int i = tid; i < n; i += nthr) {
+        const int e = idx[i];
+        if (e < 0 || e >= experts) continue;
+        atomicAdd(&s_off[e], 1);
+        if (i < mine0 + topk)
+            for (int k = 0; k < topk; ++k)
+                if (e == s_e[k] && i < mine0 + k) atomicAdd(&s_rk[k], 1);
+    }
+    __syncthreads();
+    /* exclusive scan of the counts, in place: a thread owns `chunk` consecutive experts */
+    const int chunk = (experts + nthr - 1) / nthr, b0 = tid * chunk;
+    int32_t sum = 0;
+    for (int j = 0; j < chunk; ++j)
+        if (b0 + j < experts) sum += s_off[b0 + j];
+    int32_t incl = sum;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int32_t o = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += o;
+    }
+    if (lane == 63) s_tmp[1 + wave] = incl;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) incl += s_tmp[1 + w];
+    int32_t run = incl - sum;
+    const bool writer = blockIdx.x == 0;
+    for (int j = 0; j < chunk; ++j) {
+        const int e = b0 + j;
+        if (e >= experts) break;
+        const int32_t c = s_off[e];
+        s_off[e] = run;
+        if (writer) {
+            if (il.row_off) il.row_off[e] = run;
+            if (il.incl_i32) il.incl_i32[e] = run + c;
+            if (il.counts_i64) il.counts_i64[e] = c;
+            if (il.nums_typed) il.nums_typed[e] = il.token_nums_type == 0 ? (int64_t)(run + c) : (int64_t)c;
+        }
+        run += c;
+        if (writer && e == experts - 1 && il.row_off) il.row_off[experts] = run;
+    }
+    if (tid < topk) {
+        const int e = s_e[tid];
+        const int32_t rk = (e >= 0 && e < experts && t < active) ? s_rk[tid] : -1;
+        s_rk[tid] = rk;
+        il.expand_idx[(int64_t)t * topk + tid] = rk;
+    }
+    __syncthreads();
+}
+
 /* load 16 consecutive 16-bit elements as fp32 */
 template <int XDT> __device__ __forceinline__ void load16(const uint16_t *__restrict__ p, float (&v)[16])
 {
@@ -91,15 +183,21 @@ __device__ __forceinline__ u32x4 pack16_e4m3(const float (&v)[16], float mult)
  * SLOTS = ceil(H / 16 / blockDim): 16-element segments each lane keeps in registers.
  * QM: quant flavour. SMOOTH: per-expert fp32 multipliers [E,H] (int8 only).
  */
-template <int XDT, int QM, int SLOTS, bool SMOOTH>
+template <int XDT, int QM, int SLOTS, bool SMOOTH, bool INLINE>
 __global__ void __launch_bounds__(kThreads)
 permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ topk_idx,
                      const int32_t *__restrict__ rank_in_expert, const int32_t *__restrict__ base, int base_inclusive,
-                     const float *__restrict__ smooth, int hidden, int topk, int experts, PeerRows pr)
+                     const float *__restrict__ smooth, int hidden, int topk, int experts, PeerRows pr, InlineLayout il,
+                     uint32_t *__restrict__ clear_words, int64_t clear_count)
 {
     __shared__ float red[kThreads / 64];
+    __shared__ int32_t s_off[INLINE ? kInlineMaxExperts : 1];
+    __shared__ int32_t s_e[INLINE ? kInlineMaxTopk : 1], s_rk[INLINE ? kInlineMaxTopk : 1], s_tmp[8];
     const int t = blockIdx.x;
     const int nseg = hidden / kElemsPerLane;
+    /* words the next stage wants at zero (the row maxima the int modes' first GEMM accumulates into) */
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_count; i += (int64_t)gridDim.x * blockDim.x)
+        clear_words[i] = 0u;
     float v[SLOTS][16];
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s) {
@@ -110,6 +208,23 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             for (int i = 0; i < 16; ++i) v[s][i] = 0.0f;
         }
     }
+    if constexpr (INLINE) inline_layout(topk_idx, t, topk, experts, il, s_off, s_e, s_rk, s_tmp);     /* under the row loads */
+    /* destination of pick k of this token: false if the pick is not routed (uniform across the workgroup) */
+    auto resolve = [&](int k, int &e, int64_t &row) __attribute__((always_inline)) -> bool {
+        if constexpr (INLINE) {
+            e = s_e[k];
+            const int32_t rk = s_rk[k];
+            if (rk < 0) return false;
+            row = (int64_t)s_off[e] + rk;
+            return row < pr.rows_cap;
+        } else {
+            e = topk_idx[(int64_t)t * topk + k];
+            const int rk = rank_in_expert[(int64_t)t * topk + k];
+            if (e < 0 || e >= experts || rk < 0) return false;      /* rk < 0: the layout masked this token out */
+            row = pick_row(base, base_inclusive, pr, e, rk);
+            return row >= 0;
+        }
+    };
 
     if constexpr (QM == QM_FP8) {
         /* eight consecutive lanes share one 128-column block */
@@ -128,11 +243,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         }
         const int nblk128 = hidden / 128;
         for (int k = 0; k < topk; ++k) {
-            const int e = topk_idx[(int64_t)t * topk + k];
-            const int rk = rank_in_expert[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
-            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
-            if (row < 0) continue;
+            int e;
+            int64_t row;
+            if (!resolve(k, e, row)) continue;
             uint8_t *dest = pr.dest[e / pr.e_loc];
             float *dest_scale = pr.scale[e / pr.e_loc];
 #pragma unroll
@@ -161,11 +274,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
 #pragma unroll
         for (int s = 0; s < SLOTS; ++s) q[s] = pack16_i8(v[s], sq);
         for (int k = 0; k < topk; ++k) {
-            const int e = topk_idx[(int64_t)t * topk + k];
-            const int rk = rank_in_expert[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts || rk < 0) continue;      /* rk < 0: the layout masked this token out */
-            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
-            if (row < 0) continue;
+            int e;
+            int64_t row;
+            if (!resolve(k, e, row)) continue;
             uint8_t *dest = pr.dest[e / pr.e_loc];
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
@@ -177,11 +288,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         }
     } else {
         for (int k = 0; k < topk; ++k) {
-            const int e = topk_idx[(int64_t)t * topk + k];
-            const int rk = rank_in_expert[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts || rk < 0) continue; /* uniform across the block */
-            const int64_t row = pick_row(base, base_inclusive, pr, e, rk);
-            if (row < 0) continue;
+            int e;
+            int64_t row;
+            if (!resolve(k, e, row)) continue; /* uniform across the block */
             uint8_t *dest = pr.dest[e / pr.e_loc];
             float sv[SLOTS][16];
             float amax = 0.0f;
@@ -244,24 +353,38 @@ permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ 
     }
 }
 
+/* what a permute launch does besides permuting: work out the layout itself (small batches), clear words for the next stage */
+struct PermuteExtras {
+    const InlineLayout *inline_layout;     /* null: ranks and offsets come from the layout launch */
+    uint32_t *clear_words;
+    int64_t clear_count;
+};
+
 template <int XDT, int QM, bool SMOOTH>
 int32_t launch_quant(const void *x, const int32_t *topk_idx, const int32_t *rank_in_expert, const int32_t *base,
                      int base_inclusive, const float *smooth, int64_t tokens, int64_t hidden, int64_t topk,
-                     int64_t experts, const PeerRows &pr, hipStream_t st)
+                     int64_t experts, const PeerRows &pr, const PermuteExtras &ex, hipStream_t st)
 {
     const int nseg = (int)(hidden / kElemsPerLane);
     int threads = (nseg + 63) / 64 * 64;
     if (threads > kThreads) threads = kThreads;
     const int slots = (nseg + threads - 1) / threads;
-#define ZB_LAUNCH(S)                                                                                              \
-    permute_quant_kernel<XDT, QM, S, SMOOTH><<<(unsigned)tokens, threads, 0, st>>>(                                \
+    const InlineLayout il = ex.inline_layout ? *ex.inline_layout : InlineLayout{};
+#define ZB_LAUNCH_I(S, INL)                                                                                       \
+    permute_quant_kernel<XDT, QM, S, SMOOTH, INL><<<(unsigned)tokens, threads, 0, st>>>(                           \
         (const uint16_t *)x, topk_idx, rank_in_expert, base, base_inclusive, smooth, (int)hidden, (int)topk,       \
-        (int)experts, pr)
+        (int)experts, pr, il, ex.clear_words, ex.clear_count)
+#define ZB_LAUNCH(S)                                                                                              \
+    do {                                                                                                          \
+        if (ex.inline_layout) ZB_LAUNCH_I(S, true);                                                               \
+        else ZB_LAUNCH_I(S, false);                                                                               \
+    } while (0)
     if (slots <= 1) ZB_LAUNCH(1);
     else if (slots <= 2) ZB_LAUNCH(2);
     else if (slots <= 4) ZB_LAUNCH(4);
     else return ZBALHIP_INVALID;
 #undef ZB_LAUNCH
+#undef ZB_LAUNCH_I
     return zbalhip_check_launch();
 }
 
@@ -274,13 +397,14 @@ int32_t launch_quant(const void *x, const int32_t *topk_idx, const int32_t *rank
  */
 static int32_t permute_launch(const void *x, int32_t x_dtype, const int32_t *topk_idx, const int32_t *rank_in_expert,
                               const int32_t *base, int base_inclusive, const float *smooth, int64_t tokens,
-                              int64_t hidden, int64_t topk, int64_t experts, int quant, const PeerRows &pr, hipStream_t st)
+                              int64_t hidden, int64_t topk, int64_t experts, int quant, const PeerRows &pr, hipStream_t st,
+                              const PermuteExtras &ex = PermuteExtras{})
 {
     if (x_dtype != ZDT_BF16 && x_dtype != ZDT_FP16) return ZBALHIP_INVALID;
     if (hidden <= 0 || hidden > 16 * kThreads * 4 || topk <= 0 || tokens < 0) return ZBALHIP_INVALID;
     if (tokens == 0) return ZBALHIP_OK;
     if (quant == QM_COPY) {
-        if (hidden % 8 != 0) return ZBALHIP_INVALID;
+        if (hidden % 8 != 0 || ex.inline_layout || ex.clear_count) return ZBALHIP_INVALID;
         permute_copy_kernel<<<(unsigned)tokens, kThreads, 0, st>>>((const uint16_t *)x, topk_idx, rank_in_expert, base,
                                                                  base_inclusive, (int)hidden, (int)topk, (int)experts, pr);
         return zbalhip_check_launch();
@@ -289,9 +413,9 @@ static int32_t permute_launch(const void *x, int32_t x_dtype, const int32_t *top
     const bool bf = (x_dtype == ZDT_BF16);
 #define ZB_GO(QMV, SM)                                                                                               \
     return bf ? launch_quant<ZDT_BF16, QMV, SM>(x, topk_idx, rank_in_expert, base, base_inclusive, smooth, tokens,  \
-                                                 hidden, topk, experts, pr, st)                                      \
+                                                 hidden, topk, experts, pr, ex, st)                                  \
               : launch_quant<ZDT_FP16, QMV, SM>(x, topk_idx, rank_in_expert, base, base_inclusive, smooth, tokens,  \
-                                                 hidden, topk, experts, pr, st)
+                                                 hidden, topk, experts, pr, ex, st)
     if (quant == QM_FP8) { ZB_GO(QM_FP8, false); }
     if (quant == QM_INT8_EPS) { ZB_GO(QM_INT8_EPS, false); }
     if (quant == QM_INT8_NOEPS) {
@@ -300,6 +424,13 @@ static int32_t permute_launch(const void *x, int32_t x_dtype, const int32_t *top
     }
 #undef ZB_GO
     return ZBALHIP_INVALID;
+}
+
+/* the permute kernel can work the layout out itself when the batch is this small (inline_layout above) */
+static bool layout_fits_inline(int64_t tokens, int64_t topk, int64_t experts, int quant)
+{
+    return quant != QM_COPY && tokens > 0 && tokens * topk <= kInlineMaxPicks && topk <= kInlineMaxTopk &&
+           experts <= kInlineMaxExperts;
 }
 
 /* one rank that owns every expert: all rows go to `dest` */
@@ -355,11 +486,22 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
         scratch_blocks < 1)
         return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
+    const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_NOEPS : QM_FP8);
+    if (tokens > 0 && q != QM_COPY && !dynamic_scales) return ZBALHIP_INVALID;
+    if (layout_fits_inline(tokens, topk, experts, q)) {      /* one launch: the permute kernel derives ranks and counts itself */
+        InlineLayout il = {};
+        il.tokens = (int)tokens;
+        il.token_nums_type = token_nums_type;
+        il.expand_idx = expand_idx;
+        il.incl_i32 = ep_recv_counts;
+        il.nums_typed = expert_token_nums;
+        const PermuteExtras ex = {&il, nullptr, 0};
+        return permute_launch(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk, experts, q,
+                              single_window(expand_x, dynamic_scales, experts, tokens * topk), st, ex);
+    }
     const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, token_nums_type, nullptr, expand_idx,
                                                      ep_recv_counts, nullptr, nullptr, expert_token_nums, st);
     if (rc != ZBALHIP_OK) return rc;
-    const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_NOEPS : QM_FP8);
-    if (tokens > 0 && q != QM_COPY && !dynamic_scales) return ZBALHIP_INVALID;
     return permute_launch(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk, experts, q,
                           single_window(expand_x, dynamic_scales, experts, tokens * topk), st);
 }
@@ -368,18 +510,32 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
                                                const float *smooth, const uint8_t *active_mask, int64_t tokens,
                                                int64_t hidden, int64_t topk,
                                                int64_t experts, int32_t mode, void *q1, float *xs, int32_t *expand_idx,
-                                               int64_t *counts, int32_t *row_off, int32_t *scratch,
-                                               int32_t scratch_blocks, void *stream)
+                                               int64_t *counts, int32_t *row_off, uint32_t *clear_words,
+                                               int64_t clear_count, void *stream)
 {
-    if (!counts || !row_off || !scratch) return ZBALHIP_INVALID;
+    if (!counts || !row_off || clear_count < 0 || (clear_count > 0 && !clear_words)) return ZBALHIP_INVALID;
     if (tokens > 0 && (!x || !expert_ids || !q1 || !xs || !expand_idx)) return ZBALHIP_INVALID;
-    if (experts <= 0 || experts > 1024 || topk <= 0 || tokens < 0 || (mode != 1 && mode != 2) || scratch_blocks < 1)
-        return ZBALHIP_INVALID;
+    if (experts <= 0 || experts > 1024 || topk <= 0 || tokens < 0 || (mode != 1 && mode != 2)) return ZBALHIP_INVALID;
     if (mode == 2 && smooth) return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
+    const int q = mode == 2 ? QM_FP8 : QM_INT8_NOEPS;
+    if (layout_fits_inline(tokens, topk, experts, q)) {      /* one launch: the permute kernel derives ranks and offsets itself */
+        InlineLayout il = {};
+        il.active_mask = active_mask;
+        il.tokens = (int)tokens;
+        il.token_nums_type = 1;
+        il.expand_idx = expand_idx;
+        il.row_off = row_off;
+        il.counts_i64 = counts;
+        const PermuteExtras ex = {&il, clear_words, clear_count};
+        return permute_launch(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk, experts, q,
+                              single_window(q1, xs, experts, tokens * topk), st, ex);
+    }
     const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, 1, active_mask, expand_idx, nullptr,
                                                      row_off, counts, nullptr, st);
     if (rc != ZBALHIP_OK) return rc;
-    return permute_launch(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk, experts,
-                          mode == 2 ? QM_FP8 : QM_INT8_NOEPS, single_window(q1, xs, experts, tokens * topk), st);
+    if (tokens == 0 && clear_count > 0) return zbalhip_fill_i32((int32_t *)clear_words, clear_count, 0, stream);
+    const PermuteExtras ex = {nullptr, clear_words, clear_count};
+    return permute_launch(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk, experts, q,
+                          single_window(q1, xs, experts, tokens * topk), st, ex);
 }

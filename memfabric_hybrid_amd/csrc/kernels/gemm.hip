@@ -947,7 +947,8 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
                                              void *stream)
 {
     const int w_is_list = (mode & ZBALHIP_WEIGHTS_AS_LISTS) != 0;
-    mode &= ~ZBALHIP_WEIGHTS_AS_LISTS;
+    const bool rowmax_cleared = (mode & ZBALHIP_ROWMAX_CLEARED) != 0;
+    mode &= ~(ZBALHIP_WEIGHTS_AS_LISTS | ZBALHIP_ROWMAX_CLEARED);
     if (!a || !a_scale || !w1 || !w1scale || !row_off || !q2 || !scale2) return ZBALHIP_INVALID;
     if (mode < MODE_W8A8 || mode > MODE_W4A8) return ZBALHIP_INVALID;
     if (misaligned16(a) || misaligned16(w1) || misaligned16(w1scale) || misaligned16(q2) || misaligned16(sgl_ws)) return ZBALHIP_INVALID;
@@ -964,7 +965,7 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
     if (!sgl_ws) return ZBALHIP_INVALID;
     /* the row maxima live behind the SwiGLU values in the same scratch allocation */
     p.rowmax = (uint32_t *)(sgl_ws + max_rows * (n1 / 2));
-    fill_u32_kernel<<<(unsigned)((max_rows + 255) / 256), 256, 0, st>>>(p.rowmax, max_rows, 0u);
+    if (!rowmax_cleared) fill_u32_kernel<<<(unsigned)((max_rows + 255) / 256), 256, 0, st>>>(p.rowmax, max_rows, 0u);
     if (mode == MODE_W8A8) {
         const int32_t rc = launch_dma<MODE_W8A8, true, ZDT_BF16>(p, n_tiles, st);
         if (rc != ZBALHIP_OK) return rc;
