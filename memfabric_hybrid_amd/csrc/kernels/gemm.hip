@@ -847,7 +847,14 @@ grouped_gemm_dma_kernel(GemmParams p)
         tc.expert = cur.expert;
         tc.m_tile = 0;
         tc.n_tile = cur.n_tile;
-        epilogue<MODE, GMM1, OUT_DT, RG>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane, lds_rowmax, TM);
+        /*
+         * The epilogue's lane-derived offsets are worked out afresh per tile from an opaque copy of the lane number:
+         * hoisted out of the tile loop they stay live across the K loop, spill, and every reload of a spilled
+         * register is a vector-memory operation whose wait also waits for the next tile's slab in flight.
+         */
+        int lane_e = lane;
+        asm volatile("" : "+v"(lane_e));
+        epilogue<MODE, GMM1, OUT_DT, RG>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane_e, lds_rowmax, TM);
         if (!nxt.valid) break;
         cur = nxt;
         sw_buf ^= 1;
