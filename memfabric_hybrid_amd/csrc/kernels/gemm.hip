@@ -103,8 +103,17 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
 template <int MODE, bool GMM1, int OUT_DT, int RG>
 __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &tc, f32x4 (&accf)[4][8],
                                          i32x4 (&acci)[4][8], int row_begin, int row_end, int wm, int wn, int lane,
-                                         float *lds_rowmax, int tile_rows)
+                                         float *lds_rowmax, int tile_rows, const float *es)
 {
+    /*
+     * W8A8: `es` is this tile's scales in LDS, brought there by DMA while the tile was multiplied: [0, 256) the
+     * channel scales of the tile's 256 weight rows (fp32, or 256 bf16 in the first 512 bytes), [256, 256 +
+     * tile_rows) the per-token scales of its rows. A global load here is waited for with a count that also waits
+     * for the next tile's slabs, which are already in flight (decode: 5-6 % of both GEMMs). The W4A8 mode, whose
+     * channel scales travel with the slabs, still loads its per-token scale here: its kernel has no registers to
+     * spare, and a spill costs more than the wait.
+     */
+    const float *es_row = es + 256;
     const int frag_row = lane & 15;
     const int I = p.N / 2;
     const int q8 = (lane >> 4) * 8;
@@ -115,21 +124,23 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
             const int row = row_begin + (RG * mt + wm) * 16 + frag_row;
             if (row >= row_end) continue;
             float xs = 1.0f;
-            if (MODE != MODE_FP8) xs = p.a_scale[row];
+            if (MODE == MODE_W8A8) xs = es_row[(RG * mt + wm) * 16 + frag_row];
+            else if (MODE == MODE_W4A8) xs = p.a_scale[row];
 #pragma unroll
             for (int s = 0; s < 4; ++s) {         /* sub-tiles 2s and 2s+1: eight consecutive channels from n */
-                const int n = tc.n_tile * BN + wn * 128 + s * 32 + q8;
+                const int nl = wn * 128 + s * 32 + q8;       /* within the tile */
+                const int n = tc.n_tile * BN + nl;
                 float ws[8];
                 if constexpr (MODE == MODE_W8A8) {
                     if (p.wscale_is_bf16) {
-                        const u32x4 v = *reinterpret_cast<const u32x4 *>(expert_base<uint16_t>(p.wscale, p.w_is_list, tc.expert, p.N) + n);
+                        const u32x4 v = *reinterpret_cast<const u32x4 *>(reinterpret_cast<const uint16_t *>(es) + nl);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) {
                             ws[2 * i] = zb_bf16_to_f32(v[i] & 0xffffu);
                             ws[2 * i + 1] = zb_bf16_to_f32(v[i] >> 16);
                         }
                     } else {
-                        const float *wsp = expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N) + n;
+                        const float *wsp = es + nl;
                         const f32x4 v0 = *reinterpret_cast<const f32x4 *>(wsp), v1 = *reinterpret_cast<const f32x4 *>(wsp + 4);
 #pragma unroll
                         for (int i = 0; i < 4; ++i) { ws[i] = v0[i]; ws[4 + i] = v1[i]; }
@@ -158,19 +169,17 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
 #pragma unroll
         for (int mt = 0; mt < 4; ++mt) {
             const int row = row_begin + (RG * mt + wm) * 16 + frag_row;
-            int lrow = row;
-            if (lrow > p.max_rows - 1) lrow = p.max_rows - 1;
             float xs = 1.0f;
-            if (MODE != MODE_FP8) xs = p.a_scale[lrow];
+            if (MODE == MODE_W8A8) xs = es_row[(RG * mt + wm) * 16 + frag_row];
+            else if (MODE == MODE_W4A8) xs = p.a_scale[row < p.max_rows ? row : p.max_rows - 1];
             rmax[mt] = 0.0f;
 #pragma unroll
             for (int nt = 0; nt < 4; ++nt) {
-                const int j = tc.n_tile * 128 + wn * 64 + (nt >> 1) * 32 + q8 + (nt & 1) * 4;
+                const int jl = wn * 64 + (nt >> 1) * 32 + q8 + (nt & 1) * 4;       /* within the tile's 128 SwiGLU columns */
                 float g[4], u[4];
                 if constexpr (MODE == MODE_W8A8) {
-                    const float *wsb = expert_base<float>(p.wscale, p.w_is_list, tc.expert, p.N);
-                    const f32x4 wg = *reinterpret_cast<const f32x4 *>(wsb + j);
-                    const f32x4 wu = *reinterpret_cast<const f32x4 *>(wsb + I + j);
+                    const f32x4 wg = *reinterpret_cast<const f32x4 *>(es + jl);             /* gate scales, then up scales */
+                    const f32x4 wu = *reinterpret_cast<const f32x4 *>(es + 128 + jl);
 #pragma unroll
                     for (int i = 0; i < 4; ++i) {
                         g[i] = ((float)acci[mt][nt][i] * wg[i]) * xs;
@@ -613,6 +622,34 @@ grouped_gemm_dma_kernel(GemmParams p)
             }
         }
     };
+    /*
+     * W8A8: the scales a tile's epilogue needs go to LDS by DMA as well (layout: see the epilogue), into the
+     * buffer of the tile's parity, which the fp8 mode uses for its weight block scales. Rows past the tile's end
+     * repeat its last row. Issued where the block scales are: older than every slab that follows.
+     */
+    auto issue_es = [&](const Tile &t, int buf) __attribute__((always_inline)) {
+        if (MODE != MODE_W8A8) return;
+        const uint32_t dst0 = lds_addr(lds_sw) + buf * 2048;
+        if (wave_u < TM / 64) {
+            int rel = wave_u * 64 + lane;
+            if (rel > t.last_rel) rel = t.last_rel;
+            dma4_sv(p.a_scale + t.row_begin, (uint32_t)rel * 4u, __builtin_amdgcn_readfirstlane(dst0 + 1024 + wave_u * 256));
+        }
+        if (wave_u < 4) {
+            if (GMM1) {
+                const float *wsb = expert_base<float>(p.wscale, p.w_is_list, t.expert, p.N);
+                const float *src = wave_u < 2 ? wsb + t.n_tile * 128 + wave_u * 64 : wsb + I + t.n_tile * 128 + (wave_u - 2) * 64;
+                dma4_sv(src, lane * 4u, __builtin_amdgcn_readfirstlane(dst0 + wave_u * 256));
+            } else if (!p.wscale_is_bf16) {
+                const float *wsb = expert_base<float>(p.wscale, p.w_is_list, t.expert, p.N);
+                dma4_sv(wsb + t.n_tile * BN + wave_u * 64, lane * 4u, __builtin_amdgcn_readfirstlane(dst0 + wave_u * 256));
+            } else if (wave_u < 2) {
+                const uint16_t *wsb = expert_base<uint16_t>(p.wscale, p.w_is_list, t.expert, p.N);
+                dma4_sv(reinterpret_cast<const float *>(wsb + t.n_tile * BN + wave_u * 128), lane * 4u,
+                        __builtin_amdgcn_readfirstlane(dst0 + wave_u * 256));
+            }
+        }
+    };
     /* this wave's vector-memory operations per slab: what may stay outstanding while an older slab is awaited */
     constexpr int OPS = W_PARTS + 4;
     const bool extra_op_wave = sa_wave || gs_wave;                  /* one more operation per slab: the scales */
@@ -639,6 +676,7 @@ grouped_gemm_dma_kernel(GemmParams p)
     if (!cur.valid) return;
     int sw_buf = 0;
     issue_sw(cur, sw_buf);
+    issue_es(cur, sw_buf);
 #pragma unroll
     for (int s = 0; s < NSTAGE - 1; ++s) issue(cur, s, s);        /* the host guarantees KB >= NSTAGE - 1 */
     int stage = 0;
@@ -682,7 +720,10 @@ grouped_gemm_dma_kernel(GemmParams p)
              * past this tile's first barrier now, so none of them still reads that buffer; the transfers are older
              * than every slab issued from here on, so the slab waits cover them.
              */
-            if (kb == 0 && nxt.valid) issue_sw(nxt, sw_buf ^ 1);
+            if (kb == 0 && nxt.valid) {
+                issue_sw(nxt, sw_buf ^ 1);
+                issue_es(nxt, sw_buf ^ 1);
+            }
             /*
              * That stage takes the slab NSTAGE-1 steps ahead, which may belong to the next tile. It is issued in parts,
              * spread over the first half of this step's MFMAs: a wave that pushes all of its loads at once sits in the
@@ -854,7 +895,8 @@ grouped_gemm_dma_kernel(GemmParams p)
          */
         int lane_e = lane;
         asm volatile("" : "+v"(lane_e));
-        epilogue<MODE, GMM1, OUT_DT, RG>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane_e, lds_rowmax, TM);
+        epilogue<MODE, GMM1, OUT_DT, RG>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane_e, lds_rowmax, TM,
+                                         lds_sw + sw_buf * 512);
         if (!nxt.valid) break;
         cur = nxt;
         sw_buf ^= 1;
