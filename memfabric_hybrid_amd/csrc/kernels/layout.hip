@@ -431,36 +431,38 @@ topk_route_kernel(const float *__restrict__ logits, int tokens, int experts, int
         v[j] = (e < experts) ? l[e] : -__builtin_inff();
         mx = fmaxf(mx, v[j]);
     }
-    mx = zb_wave_max(mx);
-    float sum = 0.0f;
+    mx = zb_wave_reduce_dpp<true>(mx);
+    float part = 0.0f;
 #pragma unroll
     for (int j = 0; j < PER_LANE; ++j) {
         const int e = j * 64 + lane;
-        if (e < experts) sum += zb_expf(v[j] - mx);
+        if (e < experts) part += zb_expf(v[j] - mx);
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+    const float sum = zb_wave_reduce_dpp<false>(part);
 
+    /*
+     * K rounds of arg-max, each without an LDS round trip: the largest remaining logit by a DPP reduction of the
+     * lanes' own best, then its owner by one ballot per logit slot, lowest slot and lowest lane first (the lowest
+     * expert index among equal logits, as a sequential scan would pick).
+     */
     uint32_t used = 0; /* bit j: this lane's j-th logit was picked */
     float wsum = 0.0f;
     float myw = 0.0f;  /* lane k keeps the k-th weight (topk <= 32) */
     int myidx = 0;
     for (int k = 0; k < topk; ++k) {
         float best = -__builtin_inff();
+#pragma unroll
+        for (int j = 0; j < PER_LANE; ++j) {
+            const int e = j * 64 + lane;
+            if (e < experts && !((used >> j) & 1u)) best = fmaxf(best, v[j]);
+        }
+        best = zb_wave_reduce_dpp<true>(best);
         int bidx = 0x7fffffff;
 #pragma unroll
         for (int j = 0; j < PER_LANE; ++j) {
             const int e = j * 64 + lane;
-            if (e < experts && !((used >> j) & 1u)) {
-                if (bidx == 0x7fffffff || v[j] > best) { best = v[j]; bidx = e; }
-            }
-        }
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) {
-            const float ob = __shfl_xor(best, off, 64);
-            const int oi = __shfl_xor(bidx, off, 64);
-            const bool take = (oi != 0x7fffffff) && (bidx == 0x7fffffff || ob > best || (ob == best && oi < bidx));
-            if (take) { best = ob; bidx = oi; }
+            const uint64_t owners = __ballot(e < experts && !((used >> j) & 1u) && v[j] == best);
+            if (bidx == 0x7fffffff && owners) bidx = j * 64 + (__ffsll((long long)owners) - 1);
         }
         if ((bidx & 63) == lane) used |= 1u << (bidx >> 6);
         const float p = zb_expf(best - mx) / sum;
