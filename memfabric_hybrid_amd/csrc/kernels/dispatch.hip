@@ -192,12 +192,25 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
 {
     __shared__ float red[kThreads / 64];
     __shared__ int32_t s_off[INLINE ? kInlineMaxExperts : 1];
-    __shared__ int32_t s_e[INLINE ? kInlineMaxTopk : 1], s_rk[INLINE ? kInlineMaxTopk : 1], s_tmp[8];
+    __shared__ int32_t s_e[kInlineMaxTopk], s_rk[INLINE ? kInlineMaxTopk : 1], s_tmp[8];
+    __shared__ int64_t s_row[kInlineMaxTopk];
     const int t = blockIdx.x;
     const int nseg = hidden / kElemsPerLane;
     /* words the next stage wants at zero (the row maxima the int modes' first GEMM accumulates into) */
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < clear_count; i += (int64_t)gridDim.x * blockDim.x)
         clear_words[i] = 0u;
+    /*
+     * Where the token's picks go is worked out by one lane per pick while the row is on its way (the picks' index,
+     * rank and offset loads depend on each other: done pick after pick inside the store loop they cost topk round
+     * trips to L2 per workgroup): index and rank are requested before the row, the offset after it.
+     * s_row[k] < 0: pick k is not routed.
+     */
+    const bool picker = !INLINE && threadIdx.x < topk && threadIdx.x < kInlineMaxTopk;
+    int pick_e = -1, pick_rk = -1;
+    if (picker) {
+        pick_e = topk_idx[(int64_t)t * topk + threadIdx.x];
+        pick_rk = rank_in_expert[(int64_t)t * topk + threadIdx.x];
+    }
     float v[SLOTS][16];
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s) {
@@ -208,22 +221,31 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             for (int i = 0; i < 16; ++i) v[s][i] = 0.0f;
         }
     }
-    if constexpr (INLINE) inline_layout(topk_idx, t, topk, experts, il, s_off, s_e, s_rk, s_tmp);     /* under the row loads */
+    if constexpr (INLINE) {
+        inline_layout(topk_idx, t, topk, experts, il, s_off, s_e, s_rk, s_tmp);
+        if (threadIdx.x < topk) {
+            const int32_t rk = s_rk[threadIdx.x];
+            const int64_t row = rk < 0 ? -1 : (int64_t)s_off[s_e[threadIdx.x]] + rk;
+            s_row[threadIdx.x] = row < pr.rows_cap ? row : -1;
+        }
+    } else if (picker) {
+        const bool routed = pick_e >= 0 && pick_e < experts && pick_rk >= 0;      /* rank < 0: the layout masked this token out */
+        s_e[threadIdx.x] = pick_e;
+        s_row[threadIdx.x] = routed ? pick_row(base, base_inclusive, pr, pick_e, pick_rk) : -1;
+    }
+    __syncthreads();
     /* destination of pick k of this token: false if the pick is not routed (uniform across the workgroup) */
     auto resolve = [&](int k, int &e, int64_t &row) __attribute__((always_inline)) -> bool {
-        if constexpr (INLINE) {
+        if (INLINE || k < kInlineMaxTopk) {
             e = s_e[k];
-            const int32_t rk = s_rk[k];
-            if (rk < 0) return false;
-            row = (int64_t)s_off[e] + rk;
-            return row < pr.rows_cap;
-        } else {
-            e = topk_idx[(int64_t)t * topk + k];
-            const int rk = rank_in_expert[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts || rk < 0) return false;      /* rk < 0: the layout masked this token out */
-            row = pick_row(base, base_inclusive, pr, e, rk);
+            row = s_row[k];
             return row >= 0;
         }
+        e = topk_idx[(int64_t)t * topk + k];          /* more picks per token than the table holds: one by one */
+        const int rk = rank_in_expert[(int64_t)t * topk + k];
+        if (e < 0 || e >= experts || rk < 0) return false;
+        row = pick_row(base, base_inclusive, pr, e, rk);
+        return row >= 0;
     };
 
     if constexpr (QM == QM_FP8) {
