@@ -43,15 +43,15 @@ PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # HBM bytes one GMM1 launch moves at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from two
 # `rocprofv3 --pmc` runs of this script (summary and counter calibration: profiles/moe_prefill_fp8_kernels.txt)
-GMM1_TRAFFIC_BYTES_T4096 = 2.41e9
+GMM1_TRAFFIC_BYTES_T4096 = 2.51e9
 REDUCE_TRAFFIC_BYTES = 2.416e9  # 2.0 x 1048607 KiB + 262144 KiB (profiles/reduce_8x256MiB.txt)
 
 
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--tokens", type=int, default=4096, help="development only; the reported workload is 4096")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2560)
     ap.add_argument("--workload", choices=["prefill", "decode", "qwen_w4a8", "reduce"], default="prefill",
