@@ -204,6 +204,32 @@ def test_low_latency_dispatch_combine(buf, T, H, K, E, zipf, mode):
         assert calc_diff(zo.bf16_to_f32(host(out)), zo.bf16_to_f32(x) * w.sum(1, keepdims=True)) < 1e-5
 
 
+@pytest.mark.parametrize("T,H,K,E", [
+    (512, 256, 8, 32),       # 4096 picks: the largest batch whose layout the permute kernel works out itself
+    (513, 256, 8, 32),       # one token more: layout launch + permute launch
+    (24, 512, 40, 64),       # more picks per token than the kernel's pick table holds (32)
+    (100, 256, 40, 64),      # the same past 4096 picks
+    (64, 256, 4, 1024),      # the largest expert count
+])
+@pytest.mark.parametrize("mode", ["int8", "fp8"])
+def test_low_latency_dispatch_at_the_layout_switch(buf, T, H, K, E, mode):
+    """Both ways of deriving the layout (inside the permute kernel up to 4096 picks and 32 picks per token, a layout
+    launch beyond) against the oracle, with invalid picks among the valid ones."""
+    x = bf16_normal((T, H), 31)
+    idx = distinct_topk(T, E, K, 32)
+    idx[T // 2, 1] = -1
+    idx[T - 1, K - 1] = E + 5
+    use_fp8, blk, qm = {"int8": (True, False, 1), "fp8": (True, True, 2)}[mode]
+    recv, scales, count, h = buf.low_latency_dispatch(dev(x), dev(idx), T, E, use_fp8=use_fp8, fp8_block_scale=blk)
+    rows = T * K
+    r_ex, r_sc, r_eidx, r_nums, r_counts = zo.dispatch_low_latency(x, zo.DT_BF16, idx.astype(np.int32), E, qm, rows)
+    assert np.array_equal(host(h["expand_idx"])[:rows].reshape(T, K), r_eidx)
+    assert np.array_equal(host(count), r_nums) and np.array_equal(host(h["ep_recv_count"]), r_counts)
+    total = int(r_counts[-1])
+    assert np.array_equal(host(recv).view(r_ex.dtype)[:total], r_ex[:total])
+    assert np.array_equal(host(scales).view(np.uint32).reshape(rows, -1)[:total], r_sc.view(np.uint32).reshape(rows, -1)[:total])
+
+
 def test_low_latency_token_nums_type_prefix_sum(buf, monkeypatch):
     monkeypatch.setenv("MOE_EXPERT_TOKEN_NUMS_TYPE", "0")
     T, H, K, E = 64, 256, 4, 16
