@@ -1,7 +1,8 @@
 /*
  * Weighted combine (gather-reduce): out[t,:] = round(sum_k w[t,k] * y[row(t,k),:]).
  *
- * One workgroup per output token. Each lane owns 16-byte chunks (8 elements)
+ * One workgroup per output token (small batches: per piece of a token's row,
+ * so that every CU has work). Each lane owns 16-byte chunks (8 elements)
  * of the row; for a chunk it issues the loads of up to eight picks back to
  * back so that eight 16-byte requests per lane are in flight, then folds
  * them into fp32 accumulators in pick order with a separately rounded
@@ -39,32 +40,52 @@ combine_kernel(PeerSource src, const int32_t *__restrict__ base, int base_inclus
     __shared__ float s_w[kMaxTopk];
     __shared__ int s_n;
     const int t = blockIdx.x;
-    if (threadIdx.x == 0) {
+    if (threadIdx.x < 64) {
         /*
-         * Compact the valid picks, keeping their order. A pick with a valid expert but a negative rank belongs to a
-         * token that the layout masked out (x_active_mask): such a token's output row is left as it is.
+         * One lane per pick resolves its source row (three dependent loads; done pick after pick by one lane they are
+         * topk round trips in a row, which is what a small batch waits for); the valid picks are then compacted in
+         * pick order. A pick with a valid expert but a negative rank belongs to a token that the layout masked out
+         * (x_active_mask): such a token's output row is left as it is.
          */
-        int n = 0;
-        for (int k = 0; k < topk; ++k) {
+        const int k = threadIdx.x;
+        bool keep = false, masked = false;
+        const uint16_t *row_ptr = nullptr;
+        float wk = 0.0f;
+        if (k < topk) {
             const int e = topk_idx[(int64_t)t * topk + k];
-            if (e < 0 || e >= experts) continue;
             const int32_t rk = rank_in_expert[(int64_t)t * topk + k];
-            if (rk < 0) { n = -1; break; }
-            const int slot = e * src.ranks + src.my_rank;
-            const int32_t b = base_inclusive ? (slot == 0 ? 0 : base[slot - 1]) : base[slot];
-            const int64_t row = (int64_t)b + rk;
-            if (row >= src.rows_cap) continue;            /* never read past the window */
-            s_row[n] = src.y[e / src.e_loc] + row * hidden;
-            s_w[n] = w[(int64_t)t * topk + k];
-            ++n;
+            wk = w[(int64_t)t * topk + k];
+            if (e >= 0 && e < experts) {
+                if (rk < 0) masked = true;
+                else {
+                    const int slot = e * src.ranks + src.my_rank;
+                    const int32_t b = base_inclusive ? (slot == 0 ? 0 : base[slot - 1]) : base[slot];
+                    const int64_t row = (int64_t)b + rk;
+                    if (row < src.rows_cap) {            /* never read past the window */
+                        keep = true;
+                        row_ptr = src.y[e / src.e_loc] + row * hidden;
+                    }
+                }
+            }
         }
-        s_n = n;
+        const uint64_t kept = __ballot(keep);
+        const bool any_masked = __ballot(masked) != 0;
+        if (keep && !any_masked) {
+            const int pos = __popcll(kept & ((1ull << k) - 1ull));
+            s_row[pos] = row_ptr;
+            s_w[pos] = wk;
+        }
+        if (k == 0) s_n = any_masked ? -1 : __popcll(kept);
     }
     __syncthreads();
     const int n = s_n;
     if (n < 0) return;
-    const int nchunk = hidden / 8;
-    for (int c = threadIdx.x; c < nchunk; c += blockDim.x) {
+    /* blockIdx.y: a small batch spreads each row over several workgroups, so that the whole chip takes part */
+    const int nchunk_all = hidden / 8;
+    const int per_split = (nchunk_all + gridDim.y - 1) / gridDim.y;
+    const int c_begin = blockIdx.y * per_split;
+    const int nchunk = c_begin + per_split < nchunk_all ? c_begin + per_split : nchunk_all;
+    for (int c = c_begin + threadIdx.x; c < nchunk; c += blockDim.x) {
         float acc[8];
 #pragma unroll
         for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
@@ -120,14 +141,19 @@ extern "C" int32_t zbalhip_combine(const void *const *y, int32_t ranks, int32_t 
     src.e_loc = (int)(experts / ranks);
     src.rows_cap = y_rows;
     if (tokens == 0) return ZBALHIP_OK;
-    int threads = (int)((hidden / 8 + 63) / 64 * 64);
+    /* fewer tokens than two per CU: cut the rows into pieces of at least one chunk per lane of a full workgroup */
+    int splits = 1;
+    while (tokens * splits < 512 && splits < 8 && hidden / 8 / (splits * 2) >= kThreads / 2) splits *= 2;
+    const int64_t per_split = (hidden / 8 + splits - 1) / splits;
+    int threads = (int)((per_split + 63) / 64 * 64);
     if (threads > kThreads) threads = kThreads;
+    const dim3 grid((unsigned)tokens, (unsigned)splits);
     hipStream_t st = (hipStream_t)stream;
     if (dtype == ZDT_BF16)
-        combine_kernel<ZDT_BF16><<<(unsigned)tokens, threads, 0, st>>>(src, base, base_is_inclusive, w, topk_idx, send_token_idx,
+        combine_kernel<ZDT_BF16><<<grid, threads, 0, st>>>(src, base, base_is_inclusive, w, topk_idx, send_token_idx,
                                                                      (int)hidden, (int)topk, (int)experts, (uint16_t *)out);
     else
-        combine_kernel<ZDT_FP16><<<(unsigned)tokens, threads, 0, st>>>(src, base, base_is_inclusive, w, topk_idx, send_token_idx,
+        combine_kernel<ZDT_FP16><<<grid, threads, 0, st>>>(src, base, base_is_inclusive, w, topk_idx, send_token_idx,
                                                                      (int)hidden, (int)topk, (int)experts, (uint16_t *)out);
     return zbalhip_check_launch();
 }

@@ -92,13 +92,20 @@ __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, i
         active = s_tmp[0];
     }
     const int n = active * topk, mine0 = t * topk;
-    for (int i = tid; i < n; i += nthr) {
-        const int e = idx[i];
-        if (e < 0 || e >= experts) continue;
-        atomicAdd(&s_off[e], 1);
-        if (i < mine0 + topk)
-            for (int k = 0; k < topk; ++k)
-                if (e == s_e[k] && i < mine0 + k) atomicAdd(&s_rk[k], 1);
+    /* four indices per lane are requested before the first is used: the loop is a chain of round trips to L2 otherwise */
+    for (int i0 = tid; i0 < n; i0 += 4 * nthr) {
+        int ev[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) ev[u] = i0 + u * nthr < n ? idx[i0 + u * nthr] : -1;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int e = ev[u], i = i0 + u * nthr;
+            if (e < 0 || e >= experts) continue;
+            atomicAdd(&s_off[e], 1);
+            if (i < mine0 + topk)
+                for (int k = 0; k < topk; ++k)
+                    if (e == s_e[k] && i < mine0 + k) atomicAdd(&s_rk[k], 1);
+        }
     }
     __syncthreads();
     /* exclusive scan of the counts, in place: a thread owns `chunk` consecutive experts */
