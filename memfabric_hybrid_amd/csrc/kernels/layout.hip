@@ -91,21 +91,26 @@ layout_hist_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
 /*
  * Stable ranks of the picks [p0, p1) of one block: `run[e]` holds the number of earlier picks of expert e on entry
  * and the number up to p1 on return. Picks are taken 64 per wave at a time; lanes holding the same expert find
- * each other by intersecting one ballot per index bit, and the waves of the block commit in wave order.
+ * each other by intersecting one ballot per index bit. The waves do not take turns: each leaves the size of its
+ * groups in `cnt` (one byte per wave and expert, a group has at most 64 members) and a pick's rank is the running
+ * count plus the groups of the waves before its own. Ends on a barrier.
  */
 template <typename IdxT>
 __device__ __forceinline__ void rank_picks(const IdxT *__restrict__ idx, int64_t p0, int64_t p1, int experts, int nbits,
-                                           int32_t *run, int32_t *__restrict__ send_token_idx)
+                                           int32_t *run, uint8_t *cnt /* [waves][experts rounded up to 4] */,
+                                           int32_t *__restrict__ send_token_idx)
 {
     const int np = (int)(p1 - p0);
-    const int threads = blockDim.x;
+    const int threads = blockDim.x, nwaves = threads >> 6;
     const int iters = (np + threads - 1) / threads;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
+    const int pad = (experts + 3) & ~3;
 
     for (int it = 0; it < iters; ++it) {
         const int64_t i = p0 + (int64_t)it * threads + threadIdx.x;
         int64_t e64 = (i < p1) ? (int64_t)idx[i] : -1;
+        for (int j = threadIdx.x; j < nwaves * pad / 4; j += threads) reinterpret_cast<uint32_t *>(cnt)[j] = 0u;
         const bool valid = (e64 >= 0 && e64 < experts);
         const int e = valid ? (int)e64 : 0;
         uint64_t peers = __ballot(valid);
@@ -117,15 +122,23 @@ __device__ __forceinline__ void rank_picks(const IdxT *__restrict__ idx, int64_t
         const int before = __popcll(peers & lt_mask);
         const int group = __popcll(peers);
         const bool last = valid && ((peers >> lane) >> 1) == 0; /* highest lane of its group */
-        for (int w = 0; w < (threads >> 6); ++w) {
-            if (wave == w && valid) {
-                const int32_t basev = run[e];
-                send_token_idx[i] = basev + before;
-                if (last) run[e] = basev + group;
-            }
-            __syncthreads();
+        __syncthreads();
+        if (last) cnt[wave * pad + e] = (uint8_t)group;
+        __syncthreads();
+        if (valid) {
+            int32_t basev = run[e];
+            for (int w = 0; w < wave; ++w) basev += cnt[w * pad + e];
+            send_token_idx[i] = basev + before;
+        } else if (i < p1) {
+            send_token_idx[i] = -1;
         }
-        if (!valid && i < p1) send_token_idx[i] = -1;
+        __syncthreads();
+        for (int e2 = threadIdx.x; e2 < experts; e2 += threads) {
+            int32_t sum = 0;
+            for (int w = 0; w < nwaves; ++w) sum += cnt[w * pad + e2];
+            run[e2] += sum;
+        }
+        __syncthreads();
     }
 }
 
@@ -137,6 +150,7 @@ layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
 {
     __shared__ int32_t run[ZB_MAX_EXPERTS];
     __shared__ int32_t rcnt[ZB_MAX_EXPERTS];
+    __shared__ __align__(16) uint8_t cnt[ZB_LAYOUT_THREADS / 64 * ZB_MAX_EXPERTS];
     const int b = blockIdx.x;
     for (int e = threadIdx.x; e < experts; e += blockDim.x) {
         int32_t s = 0;
@@ -149,7 +163,7 @@ layout_rank_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
     const int tok0 = b * tpb;
     int tok1 = tok0 + tpb;
     if (tok1 > tokens) tok1 = tokens;
-    rank_picks(idx, (int64_t)tok0 * topk, (int64_t)tok1 * topk, experts, nbits, run, send_token_idx);
+    rank_picks(idx, (int64_t)tok0 * topk, (int64_t)tok1 * topk, experts, nbits, run, cnt, send_token_idx);
 
     /* tokens per rank: one count per (token, rank) no matter how many of the token's picks land there */
     if (tokens_per_rank) {
@@ -189,6 +203,7 @@ layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int expe
     __shared__ int32_t run[ZB_MAX_EXPERTS];
     __shared__ int32_t wsum[ZB_FUSED_THREADS / 64];
     __shared__ int32_t s_active;
+    __shared__ __align__(16) uint8_t cnt[ZB_FUSED_THREADS / 64 * ZB_MAX_EXPERTS];
     for (int e = threadIdx.x; e < experts; e += blockDim.x) run[e] = 0;
     if (threadIdx.x == 0) s_active = 0;
     __syncthreads();
@@ -217,22 +232,30 @@ layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int expe
     const int64_t p0 = (int64_t)tok0 * topk, p1 = (int64_t)tok1 * topk;
     constexpr int PER = 16 / (int)sizeof(IdxT);      /* indices per 16-byte load */
     const int64_t nvec = ((uintptr_t)idx & 15) == 0 ? p0 / PER : 0;
-    for (int64_t v = threadIdx.x; v < nvec; v += blockDim.x) {
-        const u32x4 raw = *reinterpret_cast<const u32x4 *>(idx + v * PER);
+    /* four 16-byte loads per lane are requested before the first is counted: a chain of round trips to L2 otherwise */
+    for (int64_t v0 = threadIdx.x; v0 < nvec; v0 += 4 * (int64_t)blockDim.x) {
+        u32x4 raw[4];
 #pragma unroll
-        for (int j = 0; j < PER; ++j) {
-            int64_t e;
-            if (sizeof(IdxT) == 4) e = (int32_t)raw[j];
-            else e = (int64_t)(((uint64_t)raw[2 * j + 1] << 32) | raw[2 * j]);
-            if (e >= 0 && e < experts) atomicAdd(&run[(int)e], 1);
+        for (int u = 0; u < 4; ++u) {
+            const int64_t v = v0 + u * (int64_t)blockDim.x;
+            raw[u] = v < nvec ? *reinterpret_cast<const u32x4 *>(idx + v * PER) : u32x4{~0u, ~0u, ~0u, ~0u};
         }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int j = 0; j < PER; ++j) {
+                int64_t e;
+                if (sizeof(IdxT) == 4) e = (int32_t)raw[u][j];
+                else e = (int64_t)(((uint64_t)raw[u][2 * j + 1] << 32) | raw[u][2 * j]);
+                if (e >= 0 && e < experts) atomicAdd(&run[(int)e], 1);
+            }
     }
     for (int64_t i = nvec * PER + threadIdx.x; i < p0; i += blockDim.x) {
         const int64_t e = (int64_t)idx[i];
         if (e >= 0 && e < experts) atomicAdd(&run[(int)e], 1);
     }
     __syncthreads();
-    rank_picks(idx, p0, p1, experts, nbits, run, send_token_idx);
+    rank_picks(idx, p0, p1, experts, nbits, run, cnt, send_token_idx);
     if (blockIdx.x != gridDim.x - 1) return;
 
     /* rank_picks ends on a barrier: run[] now holds the totals */
