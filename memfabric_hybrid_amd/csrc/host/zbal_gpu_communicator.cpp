@@ -6,9 +6,12 @@
  * to a ZBALOp* launcher (:306-369 for the MoE operators, :371-438 for the
  * fused one).
  *
- * MoE operators run for a group of one rank: the rank owns all experts and
- * "peer" output buffers are the caller's local tensors. Reductions run over
- * the group's registered peer windows.
+ * Ranks are modelled on one GPU: a group's peer windows are local
+ * allocations registered per rank. Normal-mode notify, dispatch and combine
+ * and the reductions address the other ranks' buffers through that window
+ * table (the same offset in every window); a group of one needs no window.
+ * The low-latency and fused operators run for a group of one rank, which
+ * owns all experts.
  */
 #include <cstdlib>
 #include <cstring>

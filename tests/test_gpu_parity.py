@@ -151,7 +151,9 @@ def test_dispatch_fp16_input(buf):
             assert np.array_equal(host(scales)[:rows], r_scale)
 
 
-@pytest.mark.parametrize("T,H,K,E", [(256, 2048, 2, 8), (128, 7168, 8, 32), (50, 4096, 8, 128), (3, 64, 1, 2)])
+# small batches cut each row into pieces for several workgroups: 7 x 4144 gives four pieces of 130, 130, 130 and 128 chunks
+@pytest.mark.parametrize("T,H,K,E", [(256, 2048, 2, 8), (128, 7168, 8, 32), (50, 4096, 8, 128), (3, 64, 1, 2), (7, 4144, 3, 4),
+                                     (1, 16384, 8, 16)])
 def test_combine_normal_exact_and_round_trip(buf, T, H, K, E):
     x = bf16_normal((T, H), 11)
     idx = distinct_topk(T, E, K, 12)
