@@ -75,6 +75,13 @@ __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, i
 {
     const int tid = threadIdx.x, nthr = blockDim.x, lane = tid & 63, wave = tid >> 6;
     for (int e = tid; e < experts; e += nthr) s_off[e] = 0;
+    /* the first four indices of this lane are requested together with the token's own picks (no mask: every token counts) */
+    int first[4] = {-1, -1, -1, -1};
+    if (il.active_mask == nullptr) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+            if (tid + u * nthr < il.tokens * topk) first[u] = idx[tid + u * nthr];
+    }
     if (tid < topk) {
         s_e[tid] = idx[(int64_t)t * topk + tid];
         s_rk[tid] = 0;
@@ -96,7 +103,10 @@ __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, i
     for (int i0 = tid; i0 < n; i0 += 4 * nthr) {
         int ev[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) ev[u] = i0 + u * nthr < n ? idx[i0 + u * nthr] : -1;
+        for (int u = 0; u < 4; ++u) {
+            if (i0 == tid && il.active_mask == nullptr) ev[u] = first[u];
+            else ev[u] = i0 + u * nthr < n ? idx[i0 + u * nthr] : -1;
+        }
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int e = ev[u], i = i0 + u * nthr;
@@ -147,11 +157,9 @@ __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, i
     __syncthreads();
 }
 
-/* load 16 consecutive 16-bit elements as fp32 */
-template <int XDT> __device__ __forceinline__ void load16(const uint16_t *__restrict__ p, float (&v)[16])
+/* 16 consecutive 16-bit elements (two 16-byte loads) as fp32 */
+template <int XDT> __device__ __forceinline__ void cvt16(const u32x4 &a, const u32x4 &b, float (&v)[16])
 {
-    const u32x4 a = *reinterpret_cast<const u32x4 *>(p);
-    const u32x4 b = *reinterpret_cast<const u32x4 *>(p + 8);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
         v[2 * i] = zb_half_to_f32<XDT>(a[i] & 0xffffu);
@@ -218,14 +226,15 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         pick_e = topk_idx[(int64_t)t * topk + threadIdx.x];
         pick_rk = rank_in_expert[(int64_t)t * topk + threadIdx.x];
     }
-    float v[SLOTS][16];
+    /* the row is requested here and first used after the picks are resolved: the two latencies overlap */
+    u32x4 raw[SLOTS][2];
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s) {
         const int seg = s * blockDim.x + threadIdx.x;
-        if (seg < nseg) load16<XDT>(x + (int64_t)t * hidden + (int64_t)seg * 16, v[s]);
-        else {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) v[s][i] = 0.0f;
+        raw[s][0] = raw[s][1] = u32x4{0u, 0u, 0u, 0u};
+        if (seg < nseg) {
+            raw[s][0] = *reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)seg * 16);
+            raw[s][1] = *reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)seg * 16 + 8);
         }
     }
     if constexpr (INLINE) {
@@ -241,6 +250,9 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         s_row[threadIdx.x] = routed ? pick_row(base, base_inclusive, pr, pick_e, pick_rk) : -1;
     }
     __syncthreads();
+    float v[SLOTS][16];
+#pragma unroll
+    for (int s = 0; s < SLOTS; ++s) cvt16<XDT>(raw[s][0], raw[s][1], v[s]);
     /* destination of pick k of this token: false if the pick is not routed (uniform across the workgroup) */
     auto resolve = [&](int k, int &e, int64_t &row) __attribute__((always_inline)) -> bool {
         if (INLINE || k < kInlineMaxTopk) {
