@@ -350,7 +350,14 @@ struct DmaTile {
 };
 
 template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE>
-__global__ void __launch_bounds__(TM * 2, 2)      /* TM/64 x 2 waves */
+/*
+ * TM/64 x 2 waves. The second bound is waves per SIMD, i.e. the register budget: 256 registers with two waves, 512 with
+ * one. The 128-row shape has one wave per SIMD anyway; its fp8 flavour needs more than 256 registers (block-scale
+ * products beside the accumulators) and with 256 it spilled inside the K loop, where a scratch reload also waits for
+ * the slabs in flight (1.7x slower than the 256-row shape on few-row experts). The int flavours fit 256 and are
+ * a little faster compiled for it.
+ */
+__global__ void __launch_bounds__(TM * 2, (TM == 128 && MODE == MODE_FP8) ? 1 : 2)
 grouped_gemm_dma_kernel(GemmParams p)
 {
     static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8 || MODE == MODE_W4A8, "unknown mode");
