@@ -983,14 +983,34 @@ int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
 }
 
 /*
- * Shape choice from what the host knows (the row counts themselves live on the device): with at most 128 rows
- * per expert on average the GEMM is a weight-streaming job and takes the three-stage 128-row shape, which needs
- * two K slabs to fill its pipeline.
+ * Shape choice from what the host knows (the row counts themselves live on the device). With few rows per expert the
+ * GEMM is a weight-streaming job and takes the three-stage 128-row shape (which needs two K slabs to fill its
+ * pipeline); with many it needs the arithmetic intensity of the 256-row shape. Where the two meet was measured on
+ * 7168 x 4096 / 2048 x 7168 experts (W4A8: 4096 x 3072), rows per expert on average:
+ *   - few tiles (experts x channel tiles <= 1024, e.g. 32 experts): the small tiles also balance the CUs better, and
+ *     the 128-row shape stays ahead up to 384 rows (W8A8: 15 % at 256 rows, 4 % at 384, behind by 1 % at 512) and up
+ *     to 256 rows in the first fp8 GEMM (10 % at 160-192 rows, equal at 256);
+ *   - many tiles (128 or 256 experts): the shapes meet between 96 and 128 rows for fp8 (256 experts, 128 rows: the
+ *     256-row shape 6 % ahead; 96 rows: 9 % behind), and at 128-192 rows for W8A8;
+ *   - the second fp8 GEMM (16 K slabs per tile, bf16 rows out) prefers the 256-row shape from 128 rows on in both cases;
+ *   - W4A8's few-row kernel is bound by the unpack and promote instructions of its one wave per SIMD, not by the
+ *     weight stream: equal at 64 rows, the 256-row shape 2 % ahead at 96 and 17 % at 128 (a fourth stage for the
+ *     half-size packed slabs changed nothing).
  */
+template <int MODE, bool GMM1>
+inline int64_t few_rows_limit(const GemmParams &p, int n_tiles)
+{
+    if (MODE == MODE_W4A8) return 64;
+    const bool few_tiles = (int64_t)p.experts * n_tiles <= 1024;
+    if (MODE == MODE_W8A8) return few_tiles ? 384 : 128;
+    if (GMM1) return few_tiles ? 256 : 96;
+    return 96;
+}
+
 template <int MODE, bool GMM1, int OUT_DT>
 int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
 {
-    if ((int64_t)p.max_rows <= 128 * (int64_t)p.experts && p.K >= 256)
+    if ((int64_t)p.max_rows <= few_rows_limit<MODE, GMM1>(p, n_tiles) * (int64_t)p.experts && p.K >= 256)
         return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
     return launch_dma_shape<MODE, GMM1, OUT_DT, 256, 2>(p, n_tiles, st);
 }
