@@ -109,9 +109,10 @@ TILE_ORDER_COUNTS = np.array([0, 5, 256, 257, 300, 320, 384, 385, 1024, 1030, 13
 
 @pytest.mark.parametrize("N", [256, 1280])
 def test_gemms_w8a8_tile_order_with_short_tails_bit_exact(buf, N):
-    counts, K = TILE_ORDER_COUNTS, 384
+    counts, K = TILE_ORDER_COUNTS.copy(), 384
+    counts[8] = 2048                                          # more full tiles: W8A8 keeps the 128-row shape up to 384 rows per expert
     E, rows = len(counts), int(counts.sum())
-    assert rows > 128 * E                                     # so that the launcher takes the 256-row shape
+    assert rows > 384 * E                                     # so that the launcher takes the 256-row shape
     a = rng(61).integers(-127, 128, (rows, K)).astype(np.int8)
     xs = rng(62).uniform(0.005, 0.05, rows).astype(np.float32)
     w = rng(63).integers(-16, 16, (E, K, N)).astype(np.int8)
@@ -220,6 +221,36 @@ def test_gmm1_fp8(buf, E, K, N1, rows):
     assert (host(q2) != r_q2).mean() < 0.02
 
 
+# ---- either side of the launcher's shape limits -------------------------------------------------------------
+
+@pytest.mark.parametrize("rows_per_expert", [96, 97, 256, 257, 384, 385])
+def test_gemms_at_the_shape_limits(buf, rows_per_expert):
+    """The launcher picks the 128-row or the 256-row shape from rows / experts (limits 64 .. 384 by mode and GEMM):
+    the same operands either side of every limit, W8A8 bit exact and fp8 within its tolerance."""
+    E, K, N = 4, 256, 512
+    rows = rows_per_expert * E
+    counts = ragged_counts(E, rows, 7 * rows_per_expert)
+    a = rng(81).integers(-127, 128, (rows, K)).astype(np.int8)
+    xs = rng(82).uniform(0.005, 0.05, rows).astype(np.float32)
+    w = rng(83).integers(-16, 16, (E, K, N)).astype(np.int8)
+    ws = rng(84).uniform(0.0015, 0.0045, (E, N)).astype(np.float32)
+    y = gmm2(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), capi.DT_FP32, counts, K, N, 1)
+    assert np.array_equal(host(y), zo.grouped_gemm_w8a8_dequant(a, xs, w, ws, counts))
+    q2, s2, _ = gmm1(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), counts, K, N, 1)
+    r_q2, r_s2 = zo.gmm1_swiglu_quant_w8a8(a, xs, w, ws, counts)[:2]
+    assert np.array_equal(host(s2).view(np.uint32), r_s2.view(np.uint32))
+    assert np.array_equal(host(q2), r_q2)
+    fa, fsa, fw, fsw = fp8_operands(E, K, N, rows, 85)
+    y = gmm2(buf, dev(fa), dev(fsa), buf.prepack_weight(dev(fw)), dev(fsw), capi.DT_FP32, counts, K, N, 2)
+    assert_fp8_close(zo.bf16_to_f32(host(y)), zo.bf16_to_f32(zo.gmm2_fp8(fa, fsa, fw, fsw, counts)), "fp8 GEMM", FP8_GEMM_ELEM_TOL)
+    q2, s2, _ = gmm1(buf, dev(fa), dev(fsa), buf.prepack_weight(dev(fw)), dev(fsw), counts, K, N, 2)
+    r_q2, r_s2, _ = zo.gmm1_swiglu_quant_fp8(fa, fsa, fw, fsw, counts)
+    got = zo.e4m3_to_f32(host(q2)).reshape(rows, N // 256, 128) * host(s2)[:, :, None]
+    want = zo.e4m3_to_f32(r_q2).reshape(rows, N // 256, 128) * r_s2[:, :, None]
+    assert np.allclose(host(s2), r_s2, rtol=1e-4)
+    assert_requant_close(got, want, host(q2), r_q2)
+
+
 # ---- both workgroup shapes, with more tiles than workgroups ------------------------------------------------------
 
 @pytest.mark.parametrize("E,K,N,rows", [(8, 256, 2304, 8192),     # > 128 rows per expert: 256-row tiles, 2 stages, ~300 tiles
@@ -257,7 +288,8 @@ def test_gmm1_fp8_many_tiles_per_workgroup(buf, E, K, N1, rows):
 
 # ---- W4A8 ----------------------------------------------------------------------------------------------------------
 
-@pytest.mark.parametrize("E,K,N,rows", [(4, 256, 256, 300), (16, 1024, 512, 200)])
+# 64 rows per expert is the last size that takes the 128-row shape in this mode
+@pytest.mark.parametrize("E,K,N,rows", [(4, 256, 256, 300), (16, 1024, 512, 200), (4, 256, 256, 256), (4, 256, 256, 260)])
 def test_w4a8_bit_exact(buf, E, K, N, rows):
     counts = ragged_counts(E, rows, E + K)
     a = rng(41).integers(-127, 128, (rows, K)).astype(np.int8)
