@@ -799,7 +799,12 @@ grouped_gemm_dma_kernel(GemmParams p)
                     for (int nt = 0; nt < 8; ++nt) {
                         i32x8 wf_n = wf;
                         if (nt + 1 < 8) wf_n = load_w(nt + 1);
-                        if (nt < 4 && more) issue_quarter(nt);
+                        /* the 256-row fp8 loop hands the slab out in two halves (0.6 % faster, measured against quarters on one GPU; the other loops are slower that way) */
+                        if (TM == 256) {
+                            if (more && (nt == 0 || nt == 2)) { issue_quarter(nt); issue_quarter(nt + 1); }
+                        } else if (nt < 4 && more) {
+                            issue_quarter(nt);
+                        }
                         const bool second = GMM1 ? (nt >= 4) : (wn == 1);
 #pragma unroll
                         for (int mt = 0; mt < MT; ++mt) {
