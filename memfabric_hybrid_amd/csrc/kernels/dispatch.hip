@@ -226,15 +226,15 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
         pick_e = topk_idx[(int64_t)t * topk + threadIdx.x];
         pick_rk = rank_in_expert[(int64_t)t * topk + threadIdx.x];
     }
-    /* the row is requested here and first used after the picks are resolved: the two latencies overlap */
+    /* the row is requested here (streamed: it is read once) and first used after the picks are resolved: the two latencies overlap */
     u32x4 raw[SLOTS][2];
 #pragma unroll
     for (int s = 0; s < SLOTS; ++s) {
         const int seg = s * blockDim.x + threadIdx.x;
         raw[s][0] = raw[s][1] = u32x4{0u, 0u, 0u, 0u};
         if (seg < nseg) {
-            raw[s][0] = *reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)seg * 16);
-            raw[s][1] = *reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)seg * 16 + 8);
+            raw[s][0] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)seg * 16));
+            raw[s][1] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)seg * 16 + 8));
         }
     }
     if constexpr (INLINE) {
@@ -375,7 +375,7 @@ permute_copy_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ 
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const int c = c0 + u * blockDim.x + threadIdx.x;
-            if (c < nchunk) v[u] = *reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)c * 8);
+            if (c < nchunk) v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(x + (int64_t)t * hidden + (int64_t)c * 8));
         }
         for (int k = 0; k < topk; ++k) {
             const int e = topk_idx[(int64_t)t * topk + k];
