@@ -270,6 +270,14 @@ ZBALHIP_API int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, co
                              int32_t wscale_dtype, const int32_t *row_off, int64_t experts, int64_t max_rows,
                              int64_t k, int64_t n, int32_t mode, int32_t out_dtype, void *y, void *stream);
 
+/*
+ * One-time set-up of every grouped-GEMM kernel on the current GPU (each raises its dynamic-LDS limit before its
+ * first launch, which cannot be recorded into a graph). No counterpart in the reference. Optional: a launch whose
+ * kernel is still unprepared does it itself, and refuses with an error if its stream is being captured. The host
+ * layer calls it when a communicator is created.
+ */
+ZBALHIP_API int32_t zbalhip_gemm_prepare(void);
+
 #ifdef __cplusplus
 }
 #endif

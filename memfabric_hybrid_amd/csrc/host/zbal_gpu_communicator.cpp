@@ -100,6 +100,11 @@ public:
      */
     explicit GpuCommunicator(const GroupInfo &info) : Communicator(info)
     {
+        /*
+         * The grouped-GEMM kernels are set up for this GPU now, so that none of them meets its first launch inside a
+         * stream capture later. Without a usable GPU (host-only checks of the API) this fails and is left to the launches.
+         */
+        (void)zbalhip_gemm_prepare();
         const char *sw = std::getenv("ZBAL_PROF_ENABLE");
         if (!info.traced || sw == nullptr || std::atoi(sw) != 1) return;
         int64_t points = 20480;

@@ -973,40 +973,63 @@ inline unsigned grid_for(int64_t max_rows, int64_t experts, int n_tiles, int til
 }
 
 /*
- * The large-tile kernel needs more dynamic LDS than the default limit (raised once per device) and is launched
- * with one persistent workgroup per CU, or fewer when there are not that many tiles.
+ * The kernels need more dynamic LDS than the default limit: raised once per kernel instantiation and device, which
+ * cannot be recorded into a graph. zbalhip_gemm_prepare does it for every instantiation ahead of time (the host layer
+ * calls it when a communicator is created), so that no first launch falls into a stream capture; a launch that still
+ * finds its kernel unprepared does it itself, and fails with a clear error if the stream is capturing.
+ * Returns the device's CU count through n_cus.
  */
-template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE, bool WSTREAM = false>
-int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
+template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE, bool WSTREAM>
+int32_t prepare_shape(hipStream_t st, int *n_cus)
 {
     using S = DmaShape<TM, NSTAGE, MODE == MODE_W4A8 ? 64 : 128>;
     static std::mutex mu;          /* one per kernel instantiation: guards its per-device set-up below */
     static int cus[64] = {};
     const void *kern = reinterpret_cast<const void *>(&grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE, WSTREAM>);
-    int dev = 0, n_cus = 0;
+    int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ZBALHIP_RT_ERROR;
-    {
-        std::lock_guard<std::mutex> guard(mu);
-        if (cus[dev] == 0) {
-            /* the first launch on a device raises the kernel's LDS limit, which cannot be recorded into a graph */
-            hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
-            if (st != nullptr && hipStreamIsCapturing(st, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone) {
-                zbalhip_set_last_error("grouped GEMM: the first launch on a device must happen outside of a stream capture");
-                return ZBALHIP_RT_ERROR;
-            }
-            int n = 0;
-            if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return ZBALHIP_RT_ERROR;
-            if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
-                return ZBALHIP_RT_ERROR;
-            cus[dev] = n;
+    std::lock_guard<std::mutex> guard(mu);
+    if (cus[dev] == 0) {
+        hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+        if (st != nullptr && hipStreamIsCapturing(st, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone) {
+            zbalhip_set_last_error("grouped GEMM: the first launch on a device must happen outside of a stream capture");
+            return ZBALHIP_RT_ERROR;
         }
-        n_cus = cus[dev];
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) return ZBALHIP_RT_ERROR;
+        if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, S::LDS_BYTES) != hipSuccess)
+            return ZBALHIP_RT_ERROR;
+        cus[dev] = n;
     }
+    *n_cus = cus[dev];
+    return ZBALHIP_OK;
+}
+
+/* launched with one persistent workgroup per CU, or fewer when there are not that many tiles */
+template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE, bool WSTREAM = false>
+int32_t launch_dma_shape(const GemmParams &p, int n_tiles, hipStream_t st)
+{
+    using S = DmaShape<TM, NSTAGE, MODE == MODE_W4A8 ? 64 : 128>;
+    int n_cus = 0;
+    const int32_t rc = prepare_shape<MODE, GMM1, OUT_DT, TM, NSTAGE, WSTREAM>(st, &n_cus);
+    if (rc != ZBALHIP_OK) return rc;
     unsigned grid = grid_for(p.max_rows, p.experts, n_tiles, TM);
     const unsigned resident = (unsigned)(n_cus + 7) / 8 * 8;
     if (grid > resident) grid = resident;
     grouped_gemm_dma_kernel<MODE, GMM1, OUT_DT, TM, NSTAGE, WSTREAM><<<grid, S::THREADS, S::LDS_BYTES, st>>>(p);
     return zbalhip_check_launch();
+}
+
+/* every shape a launch of (MODE, GMM1, OUT_DT) can take */
+template <int MODE, bool GMM1, int OUT_DT>
+int32_t prepare_mode()
+{
+    int n = 0;
+    int32_t rc = prepare_shape<MODE, GMM1, OUT_DT, 256, 2, false>(nullptr, &n);
+    if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 128, 3, false>(nullptr, &n);
+    if constexpr (MODE != MODE_W4A8)
+        if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 128, 3, true>(nullptr, &n);
+    return rc;
 }
 
 /*
@@ -1123,4 +1146,18 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
     if (mode == MODE_FP8)
         return bf ? launch_dma<MODE_FP8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_FP8, false, ZDT_FP16>(p, n_tiles, st);
     return bf ? launch_dma<MODE_W4A8, false, ZDT_BF16>(p, n_tiles, st) : launch_dma<MODE_W4A8, false, ZDT_FP16>(p, n_tiles, st);
+}
+
+extern "C" int32_t zbalhip_gemm_prepare(void)
+{
+    int32_t rc = prepare_mode<MODE_W8A8, true, ZDT_BF16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_FP8, true, ZDT_BF16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W4A8, true, ZDT_BF16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W8A8, false, ZDT_BF16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W8A8, false, ZDT_FP16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_FP8, false, ZDT_BF16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_FP8, false, ZDT_FP16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W4A8, false, ZDT_BF16>();
+    if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W4A8, false, ZDT_FP16>();
+    return rc;
 }

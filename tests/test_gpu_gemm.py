@@ -68,6 +68,13 @@ def gmm1(buf, a, a_scale, w_packed, wscale, counts, K, N1, mode):
     return q2, s2, ws
 
 
+def test_gemm_kernels_are_prepared_ahead_of_the_first_launch(buf):
+    """Creating a communicator raises the LDS limit of every grouped-GEMM kernel variant (a first launch inside a
+    stream capture could not); the call is idempotent and succeeds on a GPU."""
+    assert capi.load().zbalhip_gemm_prepare() == 0
+    assert capi.load().zbalhip_gemm_prepare() == 0
+
+
 # ---- W8A8 --------------------------------------------------------------------------------------------------
 
 @pytest.mark.parametrize("E,K,N,rows", [(8, 1024, 2048, 512), (4, 256, 256, 300), (32, 2048, 512, 1024), (3, 128, 256, 5), (2, 512, 512, 700),
