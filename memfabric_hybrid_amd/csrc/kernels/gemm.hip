@@ -314,10 +314,16 @@ __device__ __forceinline__ const T *uniform_ptr(const T *p)
  * One LDS-DMA transfer with the address split the way the instruction wants it: a wave-uniform 64-bit base in
  * scalar registers plus a 32-bit offset per lane, and the wave's LDS destination in M0. Spelled out because
  * the compiler otherwise keeps a 64-bit vector address per transfer alive across the whole K loop.
+ *
+ * The base often reaches the asm through v_readfirstlane. A scalar register written by a vector instruction must not
+ * be read by a vector-memory instruction within five wait states, and the compiler, which inserts such waits for its
+ * own instructions, does not look inside the asm text. So the text brings them along: the move to M0 is one,
+ * `s_nop 3` the other four. (With no wait state at all the load used the register's old contents and the kernel
+ * faulted; the two states of an `s_nop 0` ran clean, but the documented figure is five.)
  */
 __device__ __forceinline__ void dma16_sv(const uint8_t *uniform_base, uint32_t lane_off, uint32_t lds_wave_addr)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(lds_wave_addr), "v"(lane_off), "s"(uniform_ptr(uniform_base))
                  : "memory", "m0");
@@ -331,7 +337,7 @@ __device__ __forceinline__ void dma16_sv(const uint8_t *uniform_base, uint32_t l
  */
 __device__ __forceinline__ void dma16_sv_nt(const uint8_t *uniform_base, uint32_t lane_off, uint32_t lds_wave_addr)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2 nt"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2 nt"
                  :
                  : "s"(lds_wave_addr), "v"(lane_off), "s"(uniform_ptr(uniform_base))
                  : "memory", "m0");
@@ -339,7 +345,7 @@ __device__ __forceinline__ void dma16_sv_nt(const uint8_t *uniform_base, uint32_
 
 __device__ __forceinline__ void dma4_sv(const float *uniform_base, uint32_t lane_off_bytes, uint32_t lds_wave_addr)
 {
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dword %1, %2"
                  :
                  : "s"(lds_wave_addr), "v"(lane_off_bytes), "s"(uniform_ptr(uniform_base))
                  : "memory", "m0");
