@@ -663,6 +663,76 @@ def test_fused_moe_rejects_bad_arguments(buf):
     assert b"pre-packed" in lib.zbal_get_last_error_msg()
 
 
+# ---- seeded random shapes ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("seed", [11, 12])
+def test_fused_moe_random_shapes(buf, seed):
+    """Forty layers per seed with shapes, expert counts, top-k, routing skew and quantisation mode drawn at random
+    (token counts around the tile edges, one expert to a hundred): int modes bit-exact, fp8 within tolerance."""
+    r = rng(seed)
+    for it in range(40):
+        mode = int(r.choice([0, 1, 2, 3]))
+        E = int(r.choice([1, 2, 3, 5, 8, 16, 17, 32, 64, 100]))
+        K = int(r.integers(1, min(8, E) + 1))
+        T = int(r.choice([1, 2, 7, 33, 64, 100, 129, 257, 300, 511, 700]))
+        H = int(r.choice([256, 512, 768, 1024, 1280]))
+        I = int(r.choice([128, 256, 384, 512]))
+        zipf = [None, 1.2, 2.0][int(r.integers(0, 3))]
+        what = "case %d: mode %d, %d tokens x %d, top-%d of %d, I = %d, zipf %s" % (it, mode, T, H, K, E, I, zipf)
+        x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 1000 * seed + it, zipf)
+        out, nums = run_fused(buf, x, ids, es, w1, s1, w2, s2, E, mode)
+        ref, counts = zo.fused_moe(x, zo.DT_BF16, ids, es, w1, s1, w2, s2, E, mode)
+        assert np.array_equal(nums, counts), what
+        if mode == 2:
+            assert_fp8_close(zo.bf16_to_f32(out), zo.bf16_to_f32(ref), what)
+        else:
+            assert np.array_equal(out, ref), what
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_w8a8_gemms_random_row_counts_bit_exact(buf, seed):
+    """Forty launches per seed of either W8A8 GEMM with the rows dealt to 1..257 experts evenly, to a few experts only,
+    in counts around the tile edges, or Zipf-skewed."""
+    r = rng(seed)
+    for it in range(40):
+        E = int(r.choice([1, 2, 3, 7, 16, 33, 64, 128, 257]))
+        K = int(r.choice([128, 256, 384, 512, 1024]))
+        N = int(r.choice([256, 512, 768, 1280]))
+        style = int(r.integers(0, 4))
+        if style == 0:
+            counts = r.multinomial(int(r.integers(1, 3000)), np.ones(E) / E)
+        elif style == 1:
+            counts = np.zeros(E, dtype=np.int64)
+            hot = r.choice(E, size=min(E, 3), replace=False)
+            counts[hot] = r.integers(1, 1500, size=len(hot))
+        elif style == 2:
+            counts = r.choice([0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 383, 384, 385, 513], size=E)
+            if counts.sum() > 6000:
+                counts = counts // 4
+        else:
+            p = 1.0 / np.arange(1, E + 1) ** 1.2
+            counts = r.multinomial(int(r.integers(1, 3000)), p / p.sum())
+        counts = counts.astype(np.int64)
+        if counts.sum() == 0:
+            counts[0] = 1
+        rows = int(counts.sum())
+        first = bool(r.integers(0, 2))
+        what = "case %d: %s, %d experts, K = %d, N = %d, counts %s" % (it, "GMM1" if first else "GMM2", E, K, N, counts.tolist()[:20])
+        a = r.integers(-127, 128, (rows, K)).astype(np.int8)
+        xs = r.uniform(0.005, 0.05, rows).astype(np.float32)
+        ws = r.uniform(0.0015, 0.0045, (E, N)).astype(np.float32)
+        if first:
+            w = r.integers(-16, 16, (E, K, N)).astype(np.int8)
+            q2, s2, _ = gmm1(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), counts, K, N, 1)
+            r_q2, r_s2 = zo.gmm1_swiglu_quant_w8a8(a, xs, w, ws, counts)[:2]
+            assert np.array_equal(host(s2).view(np.uint32), r_s2.view(np.uint32)), what
+            assert np.array_equal(host(q2), r_q2), what
+        else:
+            w = r.integers(-128, 128, (E, K, N)).astype(np.int8)
+            y = gmm2(buf, dev(a), dev(xs), buf.prepack_weight(dev(w)), dev(ws), capi.DT_FP32, counts, K, N, 1)
+            assert np.array_equal(host(y), zo.grouped_gemm_w8a8_dequant(a, xs, w, ws, counts)), what
+
+
 # ---- BASELINE configuration 1 end to end --------------------------------------------------------------------------------
 
 def test_config1_small_moe_layer(buf):
