@@ -171,6 +171,11 @@ ZBALHIP_API int32_t zbalhip_trace_free(uint64_t *host_ring);
  * allreduce.cpp:206-260): out[j] = op over p = 0..n_in-1 of in[p][j].
  * `in` is a HOST array of n_in <= ZBALHIP_MAX_REDUCE_PEERS device pointers.
  * Float types accumulate in fp32 in order p = 0..n_in-1 and round once.
+ * Every pointer must hold whole elements. 16-byte vectors are used when all
+ * pointers sit at the same offset from a 16-byte boundary (aligned buffers,
+ * or equal slices of equal windows written to a slice of the same kind; a few
+ * leading elements are then handled one by one); pointers at different
+ * offsets are reduced element by element, several times slower.
  * op is a zbal_reduce_op_t value; PROD is a true product. trace_frame != 0
  * (a zbal_profiling_name_t value of the reference,
  * zbal_comm_host_device_struct.h:27-70) records that frame around each traced

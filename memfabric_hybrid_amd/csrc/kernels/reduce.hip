@@ -193,10 +193,39 @@ __global__ void reduce_tail_kernel(ReducePtrs in, int n_in, int64_t first, int64
     else ((uint16_t *)out)[j] = (uint16_t)zb_f32_to_half<DT>(acc);
 }
 
+/* element by element over [first, count): the tail of the vector path, and the whole job when the bases disagree about their alignment */
 template <int DT, int OP>
-int32_t launch_reduce(const ReducePtrs &ptrs, int n_in, int64_t count, void *out, hipStream_t st)
+void launch_scalar(const ReducePtrs &ptrs, int n_in, int64_t first, int64_t count, void *out, hipStream_t st)
+{
+    const int64_t n = count - first;
+    if (n <= 0) return;
+    if (n <= 64) reduce_tail_kernel<DT, OP><<<1, 64, 0, st>>>(ptrs, n_in, first, count, out);
+    else reduce_tail_kernel<DT, OP><<<(unsigned)((n + 255) / 256), 256, 0, st>>>(ptrs, n_in, first, count, out);
+}
+
+/*
+ * `head` = elements in front of the first 16-byte boundary, the same for every base (0 when they are aligned), or
+ * -1 when the bases sit at different offsets from a boundary: then no vector of one lines up with a vector of the
+ * others, and the job runs element by element (correct, several times slower; reduce-scatter slices of odd length are
+ * the case it is for).
+ */
+template <int DT, int OP>
+int32_t launch_reduce(ReducePtrs ptrs, int n_in, int64_t count, void *out, int head, hipStream_t st)
 {
     constexpr int PER = Elem<DT>::per;
+    constexpr int ESZ = 16 / PER;
+    if (head < 0) {
+        launch_scalar<DT, OP>(ptrs, n_in, 0, count, out, st);
+        return zbalhip_check_launch();
+    }
+    if (head > 0) {
+        if (head > count) head = (int)count;
+        launch_scalar<DT, OP>(ptrs, n_in, 0, head, out, st);
+        for (int p = 0; p < n_in; ++p) ptrs.p[p] = (const char *)ptrs.p[p] + (size_t)head * ESZ;
+        out = (char *)out + (size_t)head * ESZ;
+        count -= head;
+        if (count == 0) return zbalhip_check_launch();
+    }
     const int64_t nvec = count / PER;
     if (nvec > 0) {
         /* one 16-byte vector per thread: measured on MI355X, short-lived workgroups stream faster (6.2 TB/s for
@@ -214,19 +243,28 @@ int32_t launch_reduce(const ReducePtrs &ptrs, int n_in, int64_t count, void *out
                 reduce_kernel<DT, OP, ZBALHIP_MAX_REDUCE_PEERS><<<(unsigned)blocks, 256, 0, st>>>(ptrs, n_in, nvec, o);
         }
     }
-    const int64_t first = nvec * PER;
-    if (first < count)
-        reduce_tail_kernel<DT, OP><<<1, 64, 0, st>>>(ptrs, n_in, first, count, out);
+    launch_scalar<DT, OP>(ptrs, n_in, nvec * PER, count, out, st);
     return zbalhip_check_launch();
 }
 
 template <int DT> int32_t dispatch_op(const ReducePtrs &ptrs, int n_in, int64_t count, int op, void *out, hipStream_t st)
 {
+    /* every base must hold whole elements; where it sits relative to a 16-byte boundary picks the path */
+    constexpr int ESZ = 16 / Elem<DT>::per;
+    const unsigned mis = (unsigned)((uintptr_t)out & 15u);
+    if (mis % ESZ) return ZBALHIP_INVALID;
+    bool same = true;
+    for (int p = 0; p < n_in; ++p) {
+        const unsigned m = (unsigned)((uintptr_t)ptrs.p[p] & 15u);
+        if (m % ESZ) return ZBALHIP_INVALID;
+        same = same && m == mis;
+    }
+    const int head = !same ? -1 : (mis ? (int)((16 - mis) / ESZ) : 0);
     switch (op) {
-        case OP_PROD: return launch_reduce<DT, OP_PROD>(ptrs, n_in, count, out, st);
-        case OP_SUM: return launch_reduce<DT, OP_SUM>(ptrs, n_in, count, out, st);
-        case OP_MAX: return launch_reduce<DT, OP_MAX>(ptrs, n_in, count, out, st);
-        case OP_MIN: return launch_reduce<DT, OP_MIN>(ptrs, n_in, count, out, st);
+        case OP_PROD: return launch_reduce<DT, OP_PROD>(ptrs, n_in, count, out, head, st);
+        case OP_SUM: return launch_reduce<DT, OP_SUM>(ptrs, n_in, count, out, head, st);
+        case OP_MAX: return launch_reduce<DT, OP_MAX>(ptrs, n_in, count, out, head, st);
+        case OP_MIN: return launch_reduce<DT, OP_MIN>(ptrs, n_in, count, out, head, st);
         default: return ZBALHIP_INVALID;
     }
 }
@@ -269,13 +307,8 @@ extern "C" int32_t zbalhip_reduce(const void *const *in, int32_t n_in, int64_t c
     ptrs.trace = trace_frame ? (unsigned long long *)trace_ring : nullptr;
     ptrs.trace_points = trace_ring ? (uint32_t)trace_points : 0;
     ptrs.trace_frame = (uint32_t)trace_frame;
-    /* the vector path needs 16-byte aligned bases */
-    bool aligned = ((uintptr_t)out & 15u) == 0;
-    for (int p = 0; p < n_in; ++p) {
+    for (int p = 0; p < n_in; ++p)
         if (!in[p]) return ZBALHIP_INVALID;
-        aligned = aligned && (((uintptr_t)in[p] & 15u) == 0);
-    }
-    if (!aligned) return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
     switch (dtype) {
         case ZDT_INT8: return dispatch_op<ZDT_INT8>(ptrs, n_in, count, op, out, st);

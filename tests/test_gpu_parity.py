@@ -271,6 +271,33 @@ def test_reduce_kernel_all_types(buf, dt, op):
         assert np.array_equal(host(out), ref), (N, n)
 
 
+@pytest.mark.parametrize("dt", [capi.DT_INT8, capi.DT_BF16, capi.DT_FP32, capi.DT_INT64])
+def test_reduce_bases_off_the_16_byte_boundary(buf, dt):
+    """Bases that hold whole elements but do not start on a 16-byte boundary: all at the same offset (a scalar head,
+    then the vector path), at different offsets (element by element), and half-element offsets (refused). Elements
+    in front of and behind the range stay untouched."""
+    lib = buf.lib
+    tdt = {capi.DT_BF16: torch.bfloat16, capi.DT_FP16: torch.float16}.get(dt)
+    for N, n, offs in ((4, 5000, [3] * 5), (3, 70001, [1, 1, 1, 0]), (8, 257, [0, 1, 2, 3, 4, 5, 6, 7, 1]), (2, 1, [1, 1, 1]),
+                       (5, 4099, [0] * 5 + [1])):
+        pad = 16
+        ins = make_reduce_inputs(dt, n + pad, N, 500 + N)
+        d_in = [dev(a, tdt) for a in ins]
+        es = d_in[0].element_size()
+        out = torch.zeros(n + pad, dtype=d_in[0].dtype, device="cuda")
+        arr = (ctypes.c_void_p * N)(*[t.data_ptr() + o * es for t, o in zip(d_in, offs)])
+        oo = offs[N]
+        assert lib.zbalhip_reduce(arr, N, n, dt, capi.REDUCE_SUM, out.data_ptr() + oo * es, 0, None, 0, capi.stream_ptr()) == 0
+        ref = zo.reduce([a[o:o + n].copy() for a, o in zip(ins, offs)], dt, capi.REDUCE_SUM)
+        got = host(out)
+        assert np.array_equal(got[oo:oo + n], ref), (N, n, offs)
+        assert not got[:oo].any() and not got[oo + n:].any()
+    if dt != capi.DT_INT8:
+        a = torch.zeros(64, dtype=torch.uint8, device="cuda")
+        arr = (ctypes.c_void_p * 1)(a.data_ptr() + 1)
+        assert lib.zbalhip_reduce(arr, 1, 4, dt, capi.REDUCE_SUM, a.data_ptr() + 32, 0, None, 0, capi.stream_ptr()) != 0
+
+
 def test_reduce_full_size_sampled_windows(buf):
     """8 buffers of 256 MiB in separate allocations, bf16 and fp32 sums: the output is checked on windows sampled at the
     ends and across the range (the reduction is element-wise, so a window needs only the same window of every input)."""
@@ -300,10 +327,12 @@ def test_reduce_scatter_and_all_reduce_over_peer_windows(buf):
     """cfg4 shape in miniature: 8 'ranks' as local windows, this rank reduces its slice of every peer's buffer."""
     from memfabric_hybrid_amd.operators import create_group, destroy_group
     lib = buf.lib
-    R, me, n = 8, 5, 6 * 2 ** 12
+    R, me = 8, 5
     comm = create_group("rs8", R, me)
     try:
-        for dt, tdt in ((capi.DT_BF16, torch.bfloat16), (capi.DT_FP32, None)):
+        # the second slice length puts this rank's slice of every window off the 16-byte boundary
+        for dt, tdt, n in ((capi.DT_BF16, torch.bfloat16, 6 * 2 ** 12), (capi.DT_FP32, None, 6 * 2 ** 12),
+                           (capi.DT_BF16, torch.bfloat16, 1001), (capi.DT_FP32, None, 333)):
             ins = make_reduce_inputs(dt, R * n, R, 300)
             wins = [dev(a, tdt) for a in ins]
             esz = wins[0].element_size()
