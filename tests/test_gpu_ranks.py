@@ -111,8 +111,19 @@ class KernelSeam:
 @pytest.mark.parametrize("api_cls", [OuterAbi, KernelSeam])
 @pytest.mark.parametrize("R,quant", [(4, capi.NO_QUANT), (4, capi.QUANT_INT8), (2, capi.QUANT_FP8_B128), (1, capi.QUANT_INT8)])
 def test_dispatch_and_combine_over_modelled_ranks(buf, R, quant, api_cls):
+    run_modelled_ranks(buf, R, quant, api_cls, 96, 4, 16, 256)
+
+
+@pytest.mark.parametrize("R,quant,T,K,E,H", [(16, capi.QUANT_INT8, 40, 8, 32, 512),       # the most ranks the tables hold
+                                             (8, capi.NO_QUANT, 1, 1, 8, 128),            # one token, one expert per rank
+                                             (2, capi.QUANT_FP8_B128, 700, 3, 6, 1024),   # more picks than one layout block ranks at once
+                                             (3, capi.NO_QUANT, 257, 8, 48, 7168)])       # odd rank count, full hidden size
+def test_modelled_ranks_other_shapes(buf, R, quant, T, K, E, H):
+    run_modelled_ranks(buf, R, quant, OuterAbi, T, K, E, H)
+
+
+def run_modelled_ranks(buf, R, quant, api_cls, T, K, E, H):
     lib = buf.lib
-    T, K, E, H = 96, 4, 16, 256
     rows_cap = R * T * K                      # what a window's receive tensors hold: every pick of every rank
     ti = capi.tensor_info
     ref = ctypes.byref
@@ -122,7 +133,7 @@ def test_dispatch_and_combine_over_modelled_ranks(buf, R, quant, api_cls):
     layout = [("counts", E * 4, torch.int32), ("recv_x", rows_cap * H * qbytes, torch.uint8),
               ("recv_scale", rows_cap * scales_per_row * 4, torch.float32), ("expert_out", rows_cap * H * 2, torch.bfloat16)]
     wins = Window.make(layout, R)
-    api = api_cls(lib, wins, "%d_%d" % (R, quant))
+    api = api_cls(lib, wins, "%d_%d_%d_%d" % (R, quant, T, H))
     try:
         # ---- every rank: layout of its own batch (counts land in its window)
         xs, idx, send_idx, w = [], [], [], []
