@@ -218,8 +218,9 @@ ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int
  * active_mask (optional, one byte per token): only the first
  * sum(mask) tokens are routed, as in the reference's TokenActiveMaskCal
  * (…swiglu_quant_multistage_workspace.h:836-863); the picks of the others get
- * expand_idx = -1, which zbalhip_combine reads as "leave this token's output
- * row alone".
+ * expand_idx = -2, which zbalhip_combine reads as "leave this token's output
+ * row alone" (-1 is a pick with an invalid expert id: it contributes nothing,
+ * but its token's row is still written).
  */
 ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids, const float *smooth,
                                     const uint8_t *active_mask,

@@ -44,8 +44,9 @@ combine_kernel(PeerSource src, const int32_t *__restrict__ base, int base_inclus
         /*
          * One lane per pick resolves its source row (three dependent loads; done pick after pick by one lane they are
          * topk round trips in a row, which is what a small batch waits for); the valid picks are then compacted in
-         * pick order. A pick with a valid expert but a negative rank belongs to a token that the layout masked out
-         * (x_active_mask): such a token's output row is left as it is.
+         * pick order. Rank -2 (or a negative rank on a valid expert id) belongs to a token that the layout masked
+         * out (x_active_mask): such a token's output row is left as it is. Rank -1 on an invalid expert id is a pick
+         * that goes nowhere: the token's row is still written, from its other picks, or as zeros if it has none.
          */
         const int k = threadIdx.x;
         bool keep = false, masked = false;
@@ -55,7 +56,8 @@ combine_kernel(PeerSource src, const int32_t *__restrict__ base, int base_inclus
             const int e = topk_idx[(int64_t)t * topk + k];
             const int32_t rk = rank_in_expert[(int64_t)t * topk + k];
             wk = w[(int64_t)t * topk + k];
-            if (e >= 0 && e < experts) {
+            if (rk == -2) masked = true;
+            else if (e >= 0 && e < experts) {
                 if (rk < 0) masked = true;
                 else {
                     const int slot = e * src.ranks + src.my_rank;

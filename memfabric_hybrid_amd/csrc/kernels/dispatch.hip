@@ -69,7 +69,10 @@ struct InlineLayout {
     int64_t *nums_typed;          /* [E] counts (type 1) or running sums (type 0) */
 };
 
-/* on return s_off[e] = rows before expert e, s_e[k] / s_rk[k] = expert and rank of pick k of token t (rank -1: not routed) */
+/*
+ * On return s_off[e] = rows before expert e, s_e[k] / s_rk[k] = expert and rank of pick k of token t. Negative ranks are
+ * not routed: -1 an invalid expert id, -2 a token past the active ones (the combine leaves such a token's row alone).
+ */
 __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, int t, int topk, int experts,
                                               const InlineLayout &il, int32_t *s_off, int32_t *s_e, int32_t *s_rk, int32_t *s_tmp)
 {
@@ -150,7 +153,7 @@ __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, i
     }
     if (tid < topk) {
         const int e = s_e[tid];
-        const int32_t rk = (e >= 0 && e < experts && t < active) ? s_rk[tid] : -1;
+        const int32_t rk = t >= active ? -2 : ((e >= 0 && e < experts) ? s_rk[tid] : -1);
         s_rk[tid] = rk;
         il.expand_idx[(int64_t)t * topk + tid] = rk;
     }

@@ -210,7 +210,9 @@ layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int expe
     /*
      * x_active_mask (one bool per token): the reference processes the first sum(mask) tokens and nothing else
      * (TokenActiveMaskCal, fused_deep_moe/gemm/kernel/...swiglu_quant_multistage_workspace.h:836-863). Picks of
-     * the other tokens get rank -1 here, which the permute and combine kernels take as "not there".
+     * the other tokens get rank -2 here: the permute kernel skips every negative rank, and the combine kernel leaves
+     * the output row of such a token alone. (-1 is a pick with an invalid expert id in a token that is routed: the
+     * combine still writes that token's row, from its other picks or as zeros.)
      */
     int active = tokens;
     if (active_mask) {
@@ -226,7 +228,7 @@ layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int expe
     int tok1 = tok0 + tpb;
     if (tok1 > tokens) tok1 = tokens;
     for (int64_t i = (int64_t)(tok0 > active ? tok0 : active) * topk + threadIdx.x; i < (int64_t)tok1 * topk; i += blockDim.x)
-        send_token_idx[i] = -1;
+        send_token_idx[i] = -2;
     if (tok0 > active) tok0 = active;
     if (tok1 > active) tok1 = active;
     const int64_t p0 = (int64_t)tok0 * topk, p1 = (int64_t)tok1 * topk;

@@ -110,9 +110,11 @@ class OperatorBuffer:
     def _ti(t, **kw):
         return ctypes.byref(capi.tensor_info(t, **kw))
 
-    def _list_ti(self, seq, num_experts, **kw):
+    def _list_ti(self, seq, num_experts, live, **kw):
         """Descriptor of a tensor list: shape and type of the stacked tensor, `data` = a device table of the
-        per-expert addresses (kept in a small cache, so repeated calls with the same tensors copy nothing)."""
+        per-expert addresses (kept in a small cache, so repeated calls with the same tensors copy nothing). The
+        descriptor holds the table's raw address only, so the table itself is appended to `live`, which the caller
+        keeps until its operator call has been issued: the cache may drop its own reference at any insertion."""
         if len(seq) != num_experts:
             raise ValueError("a tensor list needs one tensor per expert")
         first = seq[0]
@@ -121,12 +123,13 @@ class OperatorBuffer:
             if not t.is_contiguous() or t.dtype != first.dtype or t.numel() != first.numel():
                 raise ValueError("tensor-list entries must be contiguous and alike")
         key = tuple(t.data_ptr() for t in seq)
-        table = self._tables.get(key)
+        table = self._tables.pop(key, None)
         if table is None:
-            if len(self._tables) >= 64:
-                self._tables.clear()
             table = torch.tensor(key, dtype=torch.int64).to(self.device)
-            self._tables[key] = table
+        self._tables[key] = table        # most recently used last
+        while len(self._tables) > 64:
+            del self._tables[next(iter(self._tables))]
+        live.append(table)
         ti = capi.tensor_info(first, shape=(num_experts,) + per, **kw)
         ti.data = table.data_ptr()
         return ctypes.byref(ti)
@@ -301,9 +304,10 @@ class OperatorBuffer:
         token_nums = self._empty((num_experts,), torch.int64)
         wdt = {0: None, 1: None, 2: capi.DT_FP8_E4M3, 3: capi.DT_INT4X2}[quant_mode]
         null = ctypes.byref(capi.TensorInfo())
+        live = []                        # this call's address tables, referenced until the call has been issued
         if is_tensor_list:
             def wti(t, **kw):
-                return self._list_ti(t, num_experts, **kw)
+                return self._list_ti(t, num_experts, live, **kw)
         else:
             wti = self._ti
         capi.check("zbal_fused_deep_moe", self.lib.zbal_fused_deep_moe(

@@ -633,6 +633,54 @@ def test_fused_moe_tensor_list_weights(buf, mode, T):
         assert np.array_equal(host(out), ref)
 
 
+def test_fused_moe_tensor_list_tables_outlive_cache_evictions(buf):
+    """The operator layer caches the device tables of per-expert addresses and a descriptor holds a table's raw address
+    only: an eviction while a call is still collecting its four tables must not free one of them (the next table
+    would take over its memory, and the first GEMM would read its weights through the second GEMM's addresses)."""
+    T, H, K, E, I, mode = 70, 256, 4, 8, 384, 0
+    x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 150)
+    xd, idd, esd = dev(x, torch.bfloat16), dev(ids), dev(es)
+    stacked, _, _ = buf.fused_deep_moe(xd, idd, buf.prepack_weight(dev(w1)), dev(s1), buf.prepack_weight(dev(w2)),
+                                       dev(s2, torch.bfloat16), esd, E, quant_mode=mode)
+    want = host(stacked)
+    for fill in (60, 61, 62, 63, 64):
+        buf._tables.clear()
+        for i in range(fill):
+            buf._tables[("filler", i)] = torch.zeros(E, dtype=torch.int64, device="cuda")
+        def each(a, dt=None, pack=False):
+            return [buf.prepack_weight(dev(a[e:e + 1], dt)) if pack else dev(a[e:e + 1], dt).clone() for e in range(E)]
+        lists = each(w1, pack=True), each(s1), each(w2, pack=True), each(s2, torch.bfloat16)
+        out, _, _ = buf.fused_deep_moe(xd, idd, *lists, esd, E, quant_mode=mode, is_tensor_list=True)
+        assert np.array_equal(host(out), want), fill
+        assert len(buf._tables) <= 64
+    buf._tables.clear()
+
+
+@pytest.mark.parametrize("K", [1, 2])
+def test_fused_moe_active_mask_with_invalid_ids(buf, K):
+    """A token past the active ones keeps its output row even when all of its expert ids are invalid, and an active
+    token whose ids are all invalid gets a row of zeros (the combine writes the sum of no picks)."""
+    T, H, E, I, mode, active = 90, 256, 4, 128, 0, 50
+    x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, mode, 160 + K)
+    ids[3, :] = -1                   # active, nothing routed
+    ids[7, 0] = E + 2                # active, one pick dropped
+    ids[60, :] = -1                  # masked out, all ids invalid
+    ids[61, :] = E                   # the same with ids past the last expert
+    ids[62, 0] = -1
+    mask = np.zeros(T, dtype=bool)
+    mask[:active] = True
+    sentinel = torch.full((T, H), 7.0, dtype=torch.bfloat16, device="cuda")
+    out, _, nums = buf.fused_deep_moe(dev(x, torch.bfloat16), dev(ids), buf.prepack_weight(dev(w1)), dev(s1),
+                                      buf.prepack_weight(dev(w2)), dev(s2, torch.bfloat16), dev(es), E, quant_mode=mode,
+                                      x_active_mask=dev(mask), out=sentinel)
+    got = host(out)
+    assert np.array_equal(got[active:], host(torch.full((T - active, H), 7.0, dtype=torch.bfloat16)))
+    ref, counts = zo.fused_moe(x[:active], zo.DT_BF16, ids[:active], es[:active], w1, s1, w2, s2, E, mode)
+    assert np.array_equal(host(nums), counts)
+    assert np.array_equal(got[:active], ref)
+    assert not got[3].any()
+
+
 def test_fused_moe_empty_experts_and_invalid_ids(buf):
     T, H, K, E, I = 16, 256, 2, 32, 128                  # 32 picks over 32 experts: most experts are empty
     x, ids, es, w1, s1, w2, s2 = fused_inputs(T, H, K, E, I, 0, 90, zipf=1.2)
