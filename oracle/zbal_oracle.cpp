@@ -208,12 +208,18 @@ ZO_API void zo_topk_route(const float *logits, int64_t T, int64_t E, int64_t K, 
         const float *l = logits + t * E;
         float mx = l[0];
         for (int64_t e = 1; e < E; ++e) mx = std::max(mx, l[e]);
+        /*
+         * Both sums are taken in double and rounded once: the definition is "the fp32 quotient by the correctly rounded
+         * sum", which no summation order of an fp32 implementation is more than a few ulps away from (a sequential
+         * fp32 sum of a hundred equal terms, by contrast, drifts by a dozen ulps on its own).
+         */
         std::vector<float> p(E);
-        float sum = 0.0f;
-        for (int64_t e = 0; e < E; ++e) { p[e] = zo_expf_impl(l[e] - mx); sum += p[e]; }
+        double sum_d = 0.0;
+        for (int64_t e = 0; e < E; ++e) { p[e] = zo_expf_impl(l[e] - mx); sum_d += (double)p[e]; }
+        const float sum = (float)sum_d;
         for (int64_t e = 0; e < E; ++e) p[e] = p[e] / sum;
         std::vector<char> used(E, 0);
-        float wsum = 0.0f;
+        double wsum_d = 0.0;
         for (int64_t k = 0; k < K; ++k) {
             int64_t best = -1;
             for (int64_t e = 0; e < E; ++e) {
@@ -223,8 +229,9 @@ ZO_API void zo_topk_route(const float *logits, int64_t T, int64_t E, int64_t K, 
             used[best] = 1;
             topk_idx[t * K + k] = best;
             topk_w[t * K + k] = p[best];
-            wsum += p[best];
+            wsum_d += (double)p[best];
         }
+        const float wsum = (float)wsum_d;
         for (int64_t k = 0; k < K; ++k) topk_w[t * K + k] = topk_w[t * K + k] / wsum;
     }
 }

@@ -37,6 +37,19 @@ def test_router(buf, T, E, K):
     assert np.allclose(host(w), rw, rtol=1e-6, atol=0)     # north star: weights within 1e-6 relative
 
 
+@pytest.mark.parametrize("T,E,K,style", [(1000, 100, 32, "ties"), (1000, 129, 30, "ties"), (3000, 31, 24, "spread"),
+                                         (64, 1000, 28, "ties"), (100, 32, 30, "spread")])
+def test_router_many_ties_and_wide_spread(buf, T, E, K, style):
+    """Small-integer logits (dozens of equal probabilities in every sum) and logits spread over +-100 (weights down to
+    subnormal size): indices exact, normal weights within 1e-6 relative, subnormal ones within one subnormal step."""
+    g = rng(T + E + K)
+    logits = g.integers(-2, 3, (T, E)).astype(np.float32) if style == "ties" else (g.standard_normal((T, E)) * 30).astype(np.float32)
+    idx, w = buf.topk_route(dev(logits), K, idx_dtype=torch.int32)
+    ridx, rw = zo.topk_route(logits, K)
+    assert np.array_equal(host(idx), ridx)
+    assert np.allclose(host(w), rw, rtol=1e-6, atol=3e-45)
+
+
 # ---- layout / notify -------------------------------------------------------------------------
 
 @pytest.mark.parametrize("T,K,E", [(256, 2, 8), (4096, 8, 32), (16384, 8, 128), (1, 1, 1), (7, 3, 5), (1000, 6, 256),
