@@ -43,7 +43,7 @@ PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
 # HBM bytes one GMM1 launch moves at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from two
 # `rocprofv3 --pmc` runs of this script (summary and counter calibration: profiles/moe_prefill_fp8_kernels.txt)
-GMM1_TRAFFIC_BYTES_T4096 = 2.32e9
+GMM1_TRAFFIC_BYTES_T4096 = 2.29e9
 REDUCE_TRAFFIC_BYTES = 2.416e9  # 2.0 x 1048607 KiB + 262144 KiB (profiles/reduce_8x256MiB.txt)
 
 
