@@ -20,6 +20,7 @@ What differs, because this build runs one rank on one GPU:
     captured when the operator returned (the reference's is a no-op).
 """
 import os
+import weakref
 from typing import Callable, List, Optional, Tuple, Union
 
 import torch
@@ -317,15 +318,19 @@ class Buffer:
     def _packed_weight(self, w: torch.Tensor, int4: bool) -> torch.Tensor:
         if getattr(w, "zbal_prepacked", False):
             return w
+        # An entry is good only while the tensor it was made from is alive: once that tensor is freed the allocator may
+        # hand its address to other weights of the same shape, and address, shape and version would still match.
         key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
-        hit = self._packed.get(key)
-        if hit is None:
-            if len(self._packed) >= 16:
-                self._packed.clear()
+        entry = self._packed.pop(key, None)
+        if entry is not None and entry[0]() is None:
+            entry = None
+        if entry is None:
             w3 = w if w.dim() == 3 else w.unsqueeze(0)
-            hit = self.prepack_weight(w3.contiguous(), int4=int4)
-            self._packed[key] = hit
-        return hit
+            entry = (weakref.ref(w), self.prepack_weight(w3.contiguous(), int4=int4))
+        self._packed[key] = entry        # most recently used last
+        while len(self._packed) > 16:
+            del self._packed[next(iter(self._packed))]
+        return entry[1]
 
     def topk_route(self, logits: torch.Tensor, num_topk: int, idx_dtype=torch.int64):
         """Extension: softmax + top-k router; returns (topk_idx, topk_weights)."""

@@ -214,3 +214,28 @@ def test_fused_deep_moe_as_the_reference_test(buffer, bs, hidden, ffn, num_exper
             bad += 1
     assert bad <= bs * 0.05
     assert np.array_equal(host(fused_out), ref)                                  # and, in this build, bit-exact
+
+
+def test_fused_deep_moe_repacks_new_weights_at_a_reused_address(buffer):
+    """The Buffer keeps the pre-packed copies of logical weights it has seen. Weights that are freed and replaced by
+    others of the same shape usually get the same address back from the allocator: the copy of the old ones must not
+    be served for the new ones."""
+    bs, hidden, ffn, num_experts, num_topk = 32, 256, 256, 4, 2
+    torch.manual_seed(7)
+    x = (torch.rand((bs, hidden), device="cuda") * 10 - 5).to(torch.bfloat16)
+    ids = torch.randint(0, num_experts, (bs, num_topk), dtype=torch.int32, device="cuda")
+    es = torch.rand((bs, num_topk), dtype=torch.float32, device="cuda")
+    g1_s = (torch.rand((num_experts, ffn), dtype=torch.float32, device="cuda") * 0.003 + 0.0015).contiguous()
+    g2_s = (torch.rand((num_experts, hidden), dtype=torch.float32, device="cuda") * 0.003 + 0.0015).to(torch.bfloat16)
+    seen = set()
+    for round_ in range(3):
+        g1_w = torch.randint(-16, 16, (num_experts, hidden, ffn), dtype=torch.int8, device="cuda")
+        g2_w = torch.randint(-16, 16, (num_experts, ffn // 2, hidden), dtype=torch.int8, device="cuda")
+        seen.add((g1_w.data_ptr(), g2_w.data_ptr()))
+        out, nums = buffer.fused_deep_moe(x=x, topk_idx=ids, gmm1_permuted_weight=g1_w, gmm1_permuted_weight_scale=g1_s,
+                                          gmm2_weight=g2_w, gmm2_weight_scale=g2_s, topk_weights=es, num_experts=num_experts)
+        ref, _ = zo.fused_moe(host(x), zo.DT_BF16, host(ids), host(es), host(g1_w), host(g1_s), host(g2_w), host(g2_s),
+                              num_experts, 0)
+        assert np.array_equal(host(out), ref), round_
+        del g1_w, g2_w, out
+    assert len(seen) < 3          # the allocator did hand an address out again, or the test shows nothing
