@@ -111,7 +111,9 @@ ZBALHIP_API int32_t zbalhip_dispatch_normal(const void *x, int32_t x_dtype, cons
  * Replaces ZBALOpCombineNormal (zbal_npu_operators.h:64-68; kernel
  * combine_normal.h:398-494): out[t] = round(sum_k fp32(row) * w), multiply
  * and add rounded separately, k ascending, invalid ids skipped; a token with
- * a valid id but send_token_idx < 0 is not written at all. y is a HOST array
+ * send_token_idx = -2 on any pick (or a valid id with a negative
+ * send_token_idx) is not written at all: that is how the fused operator's
+ * layout marks the tokens past the active ones. y is a HOST array
  * of `ranks` device pointers (the windows the rows were dispatched to, y_rows
  * rows each; a row past that is skipped); the row of a pick of expert e is
  * row base[e * ranks + my_rank] + send_token_idx of window e / (experts /
