@@ -18,9 +18,6 @@ CSRC = os.path.join(PKG, "csrc")
 OBJ = os.path.join(CSRC, "_obj")
 LIB_DIR = os.path.join(PKG, "lib")
 LIB = os.path.join(LIB_DIR, "libzbal.so")
-# stand-alone measurement program (not part of the library): ceilings of the fp8 GEMM's main loop, piece by piece
-PROBE_SRC = os.path.join(CSRC, "probe", "gemm_ceiling_probe.hip")
-PROBE = os.path.join(LIB_DIR, "gemm_ceiling_probe")
 ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 KERNELS = ["layout", "dispatch", "combine", "reduce", "prepack", "gemm"]
@@ -75,9 +72,6 @@ def build_library(force=False, verbose=False):
         objs.append(obj)
         if force or not _newer(obj, [src] + hdrs):
             jobs.append(["g++"] + HOST_FLAGS + INCLUDES + ["-c", src, "-o", obj])
-    if force or not _newer(PROBE, [PROBE_SRC]):
-        jobs.append([os.path.join(ROCM, "bin", "hipcc"), "--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off",
-                     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-o", PROBE, PROBE_SRC])
     with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, max(1, len(jobs)))) as ex:
         for out in ex.map(_run, jobs):
             if verbose and out.strip():
