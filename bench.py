@@ -214,6 +214,7 @@ def bench_moe(args, torch, np, capi, buf, workload):
     off = {k: int(v) for k, v in plan_workspace(lib, T, H, K, E, N1, mode).items()}
     base = ws.data_ptr()
     q1, xs, eidx, row_off, q2, sc2, y = (base + off[k] for k in ("q1", "xs", "expand_idx", "row_off", "q2", "scale2", "y"))
+    lscratch = base + off["layout_scratch"]
     sgl = base + off["sgl"] if mode != 2 else None
     rowmax = sgl + rows * I * 4 if sgl else None      # int modes: row maxima behind the fp32 SwiGLU values; the permute launch clears them
     names = ["route", "permute_quant", "gmm1_swiglu_quant", "gmm2_dequant", "combine"]
@@ -227,7 +228,7 @@ def bench_moe(args, torch, np, capi, buf, workload):
         evs[1].record()
         capi.check("permute", lib.zbalhip_fused_permute_quant(x.data_ptr(), capi.DT_BF16, ids32.data_ptr(), None, None, T, H, K, E,
                                                               2 if mode == 2 else 1, q1, xs, eidx, nums.data_ptr(), row_off,
-                                                              rowmax, rows if rowmax else 0, st))
+                                                              rowmax, rows if rowmax else 0, lscratch, 50, st))
         evs[2].record()
         capi.check("gmm1", lib.zbalhip_gmm1_swiglu_quant(q1, xs, w1.data_ptr(), s1.data_ptr(), row_off, E, rows, H, N1,
                                                          mode | (capi.ROWMAX_CLEARED if rowmax else 0),

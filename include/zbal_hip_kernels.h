@@ -217,6 +217,13 @@ ZBALHIP_API int32_t zbalhip_weight_prepack(const void *src, int64_t experts, int
  * the int modes' first GEMM accumulates into, so that it needs no fill launch
  * of its own (ZBALHIP_ROWMAX_CLEARED). With at most 4096 picks (tokens x topk)
  * the permute kernel works the layout out itself and the stage is one launch.
+ * Larger batches: when `scratch` holds scratch_blocks x experts int32
+ * (scratch_blocks >= 1; up to one block per 1024 picks ranks faster) and there
+ * are at most 256 experts, the layout launch in front of the permute launch
+ * only ranks the picks within token ranges and leaves one histogram per range
+ * there; the permute workgroups derive offsets from those themselves while
+ * their rows are in flight. Otherwise (scratch_blocks = 0) the layout launch
+ * does all of it.
  * active_mask (optional, one byte per token): only the first
  * sum(mask) tokens are routed, as in the reference's TokenActiveMaskCal
  * (…swiglu_quant_multistage_workspace.h:836-863); the picks of the others get
@@ -228,7 +235,8 @@ ZBALHIP_API int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, 
                                     const uint8_t *active_mask,
                                     int64_t tokens, int64_t hidden, int64_t topk, int64_t experts, int32_t mode,
                                     void *q1, float *xs, int32_t *expand_idx, int64_t *counts, int32_t *row_off,
-                                    uint32_t *clear_words, int64_t clear_count, void *stream);
+                                    uint32_t *clear_words, int64_t clear_count, int32_t *scratch, int32_t scratch_blocks,
+                                    void *stream);
 
 /*
  * OR-ed into `mode` of the two grouped GEMMs: `w1`/`w2` and their scales are

@@ -637,6 +637,7 @@ public:
         float *xs = (float *)(base + ws.xs);
         int32_t *expandIdx = (int32_t *)(base + ws.expand_idx);
         int32_t *rowOff = (int32_t *)(base + ws.row_off);
+        int32_t *layoutScratch = (int32_t *)(base + ws.layout_scratch);   /* per-block histograms of the large-batch layout */
         void *q2 = base + ws.q2;
         float *scale2 = (float *)(base + ws.scale2);
         float *sgl = mode == 2 ? nullptr : (float *)(base + ws.sgl);
@@ -649,7 +650,8 @@ public:
         if (T == 0) { /* nothing routed: counts are zero */
             return Launched(op, zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth,
                                                             nullptr, 0, H, K, E, qmode, q1, xs, expandIdx,
-                                                            (int64_t *)expertTokenNums->data, rowOff, nullptr, 0, stream));
+                                                            (int64_t *)expertTokenNums->data, rowOff, nullptr, 0, nullptr, 0,
+                                                            stream));
         }
         int32_t rc = 0;
         if (shared) {
@@ -665,7 +667,8 @@ public:
             if (rc != 0) return Launched(op, rc);
             /* with x_active_mask the shared expert, too, sees only the first sum(mask) tokens (TokenActiveMaskCal) */
             rc = zbalhip_fused_permute_quant(x->data, x->dataType, zeroIds, shareSmooth, activeMask, T, H, 1, 1, qmode, q1, xs, expandIdx,
-                                             shareCount, rowOff, sgl ? (uint32_t *)(sgl + T * SI) : nullptr, sgl ? T : 0, stream);
+                                             shareCount, rowOff, sgl ? (uint32_t *)(sgl + T * SI) : nullptr, sgl ? T : 0,
+                                             layoutScratch, ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
             if (rc != 0) return Launched(op, rc);
             rc = zbalhip_gmm1_swiglu_quant(q1, xs, shareGmm1Weight->data, shareGmm1Scale->data, rowOff, 1, T, H, SN1,
                                            mode | clearedFlag, q2, scale2, sgl, stream);
@@ -676,7 +679,8 @@ public:
         }
         rc = zbalhip_fused_permute_quant(x->data, x->dataType, (const int32_t *)expertIds->data, smooth, activeMask, T, H, K, E,
                                          qmode, q1, xs, expandIdx, (int64_t *)expertTokenNums->data, rowOff,
-                                         sgl ? (uint32_t *)(sgl + rows * I) : nullptr, sgl ? rows : 0, stream);
+                                         sgl ? (uint32_t *)(sgl + rows * I) : nullptr, sgl ? rows : 0, layoutScratch,
+                                         ZBALHIP_LAYOUT_MAX_BLOCKS, stream);
         if (rc != 0) return Launched(op, rc);
         rc = zbalhip_gmm1_swiglu_quant(q1, xs, gmm1Weight->data, gmm1Scale->data, rowOff, E, rows, H, N1,
                                        gemmMode | clearedFlag, q2, scale2, sgl, stream);

@@ -12,6 +12,10 @@
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
 
+int32_t zbalhip_layout_ranges_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
+                                       const uint8_t *active_mask, int32_t *send_token_idx, int32_t *hist, int nblk,
+                                       int tokens_per_block, hipStream_t st);
+
 int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
                                       int32_t token_nums_type, const uint8_t *active_mask, int32_t *send_token_idx,
                                       int32_t *incl_i32, int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed,
@@ -160,6 +164,76 @@ __device__ __forceinline__ void inline_layout(const int32_t *__restrict__ idx, i
     __syncthreads();
 }
 
+/*
+ * Large batches: the layout launch in front of the permute only ranks the picks within token ranges and leaves one
+ * histogram per range (layout_ranges_kernel); what is left of the layout -- how many picks of an expert the ranges
+ * before a token's own hold, and the experts' first rows -- every permute workgroup works out for itself from that
+ * small table while its row is on its way from HBM: no workgroup of either launch waits for another, and the layout
+ * launch is a third of what it was. Workgroup 0 also writes the offsets and counts the stages after the permute read.
+ */
+constexpr int kTableMaxEntries = 2048;        /* ranges x experts */
+constexpr int kTableMaxExperts = 256;         /* one expert per thread in the scan */
+
+struct RangeTable {
+    const int32_t *hist;          /* [ranges][experts] */
+    int ranges, tokens_per_range;
+    int32_t *expand_idx;          /* [T, K]: in, the rank within the range; out, the rank within the expert */
+    int32_t *row_off;             /* [E + 1] */
+    int64_t *counts_i64;          /* [E] */
+};
+
+constexpr int kTablePerThread = kTableMaxEntries / kThreads;
+
+/* the table's entries tid, tid + kThreads, ...: requested before the row, so that they arrive first (a wave's loads return in order) */
+__device__ __forceinline__ void table_request(const RangeTable &rt, int experts, int32_t (&tabv)[kTablePerThread])
+{
+    const int n = rt.ranges * experts;
+#pragma unroll
+    for (int j = 0; j < kTablePerThread; ++j) {
+        const int i = j * kThreads + (int)threadIdx.x;
+        tabv[j] = i < n ? rt.hist[i] : 0;
+    }
+}
+
+/* On return s_first[e] = first row of expert e, s_before[e] = picks of expert e in the ranges before `range`. */
+__device__ __forceinline__ void table_layout(const RangeTable &rt, const int32_t (&tabv)[kTablePerThread], int range,
+                                             int experts, bool writer, int32_t *s_tab, int32_t *s_first, int32_t *s_before,
+                                             int32_t *s_tmp)
+{
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int j = 0; j < kTablePerThread; ++j) s_tab[j * kThreads + tid] = tabv[j];
+    __syncthreads();
+    int32_t c = 0;
+    if (tid < experts) {
+        int32_t bef = 0;
+        for (int r = 0; r < rt.ranges; ++r) {
+            const int32_t v = s_tab[r * experts + tid];
+            c += v;
+            if (r < range) bef += v;
+        }
+        s_before[tid] = bef;
+    }
+    int32_t incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int32_t o = __shfl_up(incl, off, 64);
+        if (lane >= off) incl += o;
+    }
+    if (lane == 63) s_tmp[wave] = incl;
+    __syncthreads();
+    for (int w = 0; w < wave; ++w) incl += s_tmp[w];
+    if (tid < experts) {
+        s_first[tid] = incl - c;
+        if (writer) {
+            rt.row_off[tid] = incl - c;
+            if (rt.counts_i64) rt.counts_i64[tid] = c;
+            if (tid == experts - 1) rt.row_off[experts] = incl;
+        }
+    }
+    __syncthreads();
+}
+
 /* 16 consecutive 16-bit elements (two 16-byte loads) as fp32 */
 template <int XDT> __device__ __forceinline__ void cvt16(const u32x4 &a, const u32x4 &b, float (&v)[16])
 {
@@ -201,15 +275,19 @@ __device__ __forceinline__ u32x4 pack16_e4m3(const float (&v)[16], float mult)
  * SLOTS = ceil(H / 16 / blockDim): 16-element segments each lane keeps in registers.
  * QM: quant flavour. SMOOTH: per-expert fp32 multipliers [E,H] (int8 only).
  */
-template <int XDT, int QM, int SLOTS, bool SMOOTH, bool INLINE>
+enum { LM_GIVEN = 0, LM_INLINE = 1, LM_TABLE = 2 };     /* where ranks and offsets come from */
+
+template <int XDT, int QM, int SLOTS, bool SMOOTH, int LM>
 __global__ void __launch_bounds__(kThreads)
 permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__ topk_idx,
                      const int32_t *__restrict__ rank_in_expert, const int32_t *__restrict__ base, int base_inclusive,
                      const float *__restrict__ smooth, int hidden, int topk, int experts, PeerRows pr, InlineLayout il,
-                     uint32_t *__restrict__ clear_words, int64_t clear_count)
+                     RangeTable rt, uint32_t *__restrict__ clear_words, int64_t clear_count)
 {
+    constexpr bool INLINE = LM == LM_INLINE, TABLE = LM == LM_TABLE;
     __shared__ float red[kThreads / 64];
-    __shared__ int32_t s_off[INLINE ? kInlineMaxExperts : 1];
+    __shared__ int32_t s_off[INLINE ? kInlineMaxExperts : (TABLE ? kTableMaxExperts : 1)];
+    __shared__ int32_t s_before[TABLE ? kTableMaxExperts : 1], s_tab[TABLE ? kTableMaxEntries : 1];
     __shared__ int32_t s_e[kInlineMaxTopk], s_rk[INLINE ? kInlineMaxTopk : 1], s_tmp[8];
     __shared__ int64_t s_row[kInlineMaxTopk];
     const int t = blockIdx.x;
@@ -227,8 +305,10 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
     int pick_e = -1, pick_rk = -1;
     if (picker) {
         pick_e = topk_idx[(int64_t)t * topk + threadIdx.x];
-        pick_rk = rank_in_expert[(int64_t)t * topk + threadIdx.x];
+        pick_rk = TABLE ? rt.expand_idx[(int64_t)t * topk + threadIdx.x] : rank_in_expert[(int64_t)t * topk + threadIdx.x];
     }
+    int32_t tabv[TABLE ? kTablePerThread : 1];
+    if constexpr (TABLE) table_request(rt, experts, tabv);
     /* the row is requested here (streamed: it is read once) and first used after the picks are resolved: the two latencies overlap */
     u32x4 raw[SLOTS][2];
 #pragma unroll
@@ -246,6 +326,19 @@ permute_quant_kernel(const uint16_t *__restrict__ x, const int32_t *__restrict__
             const int32_t rk = s_rk[threadIdx.x];
             const int64_t row = rk < 0 ? -1 : (int64_t)s_off[s_e[threadIdx.x]] + rk;
             s_row[threadIdx.x] = row < pr.rows_cap ? row : -1;
+        }
+    } else if constexpr (TABLE) {
+        table_layout(rt, tabv, t / rt.tokens_per_range, experts, t == 0, s_tab, s_off, s_before, s_tmp);
+        if (picker) {
+            int64_t row = -1;
+            if (pick_e >= 0 && pick_e < experts && pick_rk >= 0) {       /* rank < 0: the layout masked this token out */
+                const int32_t rk = s_before[pick_e] + pick_rk;
+                rt.expand_idx[(int64_t)t * topk + threadIdx.x] = rk;       /* the rank within the expert: what the combine reads */
+                row = (int64_t)s_off[pick_e] + rk;
+                if (row >= pr.rows_cap) row = -1;
+            }
+            s_e[threadIdx.x] = pick_e;
+            s_row[threadIdx.x] = row;
         }
     } else if (picker) {
         const bool routed = pick_e >= 0 && pick_e < experts && pick_rk >= 0;      /* rank < 0: the layout masked this token out */
@@ -402,6 +495,7 @@ struct PermuteExtras {
     const InlineLayout *inline_layout;     /* null: ranks and offsets come from the layout launch */
     uint32_t *clear_words;
     int64_t clear_count;
+    const RangeTable *range_table;         /* non-null: ranks within token ranges + the ranges' histograms (large batches) */
 };
 
 template <int XDT, int QM, bool SMOOTH>
@@ -412,16 +506,19 @@ int32_t launch_quant(const void *x, const int32_t *topk_idx, const int32_t *rank
     const int nseg = (int)(hidden / kElemsPerLane);
     int threads = (nseg + 63) / 64 * 64;
     if (threads > kThreads) threads = kThreads;
+    if (ex.range_table) threads = kThreads;       /* the table's scan gives every expert a thread */
     const int slots = (nseg + threads - 1) / threads;
     const InlineLayout il = ex.inline_layout ? *ex.inline_layout : InlineLayout{};
-#define ZB_LAUNCH_I(S, INL)                                                                                       \
-    permute_quant_kernel<XDT, QM, S, SMOOTH, INL><<<(unsigned)tokens, threads, 0, st>>>(                           \
+    const RangeTable rt = ex.range_table ? *ex.range_table : RangeTable{};
+#define ZB_LAUNCH_I(S, LMV)                                                                                       \
+    permute_quant_kernel<XDT, QM, S, SMOOTH, LMV><<<(unsigned)tokens, threads, 0, st>>>(                           \
         (const uint16_t *)x, topk_idx, rank_in_expert, base, base_inclusive, smooth, (int)hidden, (int)topk,       \
-        (int)experts, pr, il, ex.clear_words, ex.clear_count)
+        (int)experts, pr, il, rt, ex.clear_words, ex.clear_count)
 #define ZB_LAUNCH(S)                                                                                              \
     do {                                                                                                          \
-        if (ex.inline_layout) ZB_LAUNCH_I(S, true);                                                               \
-        else ZB_LAUNCH_I(S, false);                                                                               \
+        if (ex.inline_layout) ZB_LAUNCH_I(S, LM_INLINE);                                                          \
+        else if (ex.range_table) ZB_LAUNCH_I(S, LM_TABLE);                                                        \
+        else ZB_LAUNCH_I(S, LM_GIVEN);                                                                            \
     } while (0)
     if (slots <= 1) ZB_LAUNCH(1);
     else if (slots <= 2) ZB_LAUNCH(2);
@@ -539,7 +636,7 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
         il.expand_idx = expand_idx;
         il.incl_i32 = ep_recv_counts;
         il.nums_typed = expert_token_nums;
-        const PermuteExtras ex = {&il, nullptr, 0};
+        const PermuteExtras ex = {&il, nullptr, 0, nullptr};
         return permute_launch(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk, experts, q,
                               single_window(expand_x, dynamic_scales, experts, tokens * topk), st, ex);
     }
@@ -555,12 +652,13 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
                                                int64_t hidden, int64_t topk,
                                                int64_t experts, int32_t mode, void *q1, float *xs, int32_t *expand_idx,
                                                int64_t *counts, int32_t *row_off, uint32_t *clear_words,
-                                               int64_t clear_count, void *stream)
+                                               int64_t clear_count, int32_t *scratch, int32_t scratch_blocks, void *stream)
 {
     if (!counts || !row_off || clear_count < 0 || (clear_count > 0 && !clear_words)) return ZBALHIP_INVALID;
     if (tokens > 0 && (!x || !expert_ids || !q1 || !xs || !expand_idx)) return ZBALHIP_INVALID;
     if (experts <= 0 || experts > 1024 || topk <= 0 || tokens < 0 || (mode != 1 && mode != 2)) return ZBALHIP_INVALID;
     if (mode == 2 && smooth) return ZBALHIP_INVALID;
+    if (scratch_blocks < 0 || (scratch_blocks > 0 && !scratch)) return ZBALHIP_INVALID;
     hipStream_t st = (hipStream_t)stream;
     const int q = mode == 2 ? QM_FP8 : QM_INT8_NOEPS;
     if (layout_fits_inline(tokens, topk, experts, q)) {      /* one launch: the permute kernel derives ranks and offsets itself */
@@ -571,15 +669,34 @@ extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, c
         il.expand_idx = expand_idx;
         il.row_off = row_off;
         il.counts_i64 = counts;
-        const PermuteExtras ex = {&il, clear_words, clear_count};
+        const PermuteExtras ex = {&il, clear_words, clear_count, nullptr};
         return permute_launch(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk, experts, q,
+                              single_window(q1, xs, experts, tokens * topk), st, ex);
+    }
+    /* large batches with room for the ranges' histograms: a short layout launch, the rest of the layout inside the permute launch */
+    int64_t ranges = (tokens * topk + 1023) / 1024;
+    if (ranges > scratch_blocks) ranges = scratch_blocks;
+    if (ranges > kTableMaxEntries / experts) ranges = kTableMaxEntries / experts;
+    if (tokens > 0 && ranges >= 1 && experts <= kTableMaxExperts && topk <= kInlineMaxTopk && tokens * topk <= 0x7fffffff) {
+        RangeTable rt = {};
+        rt.tokens_per_range = (int)((tokens + ranges - 1) / ranges);
+        rt.ranges = (int)((tokens + rt.tokens_per_range - 1) / rt.tokens_per_range);
+        rt.hist = scratch;
+        rt.expand_idx = expand_idx;
+        rt.row_off = row_off;
+        rt.counts_i64 = counts;
+        const int32_t rc = zbalhip_layout_ranges_internal(expert_ids, tokens, experts, topk, active_mask, expand_idx, scratch,
+                                                          rt.ranges, rt.tokens_per_range, st);
+        if (rc != ZBALHIP_OK) return rc;
+        const PermuteExtras ex = {nullptr, clear_words, clear_count, &rt};
+        return permute_launch(x, x_dtype, expert_ids, nullptr, nullptr, 0, smooth, tokens, hidden, topk, experts, q,
                               single_window(q1, xs, experts, tokens * topk), st, ex);
     }
     const int32_t rc = zbalhip_layout_fused_internal(expert_ids, tokens, experts, topk, 1, active_mask, expand_idx, nullptr,
                                                      row_off, counts, nullptr, st);
     if (rc != ZBALHIP_OK) return rc;
     if (tokens == 0 && clear_count > 0) return zbalhip_fill_i32((int32_t *)clear_words, clear_count, 0, stream);
-    const PermuteExtras ex = {nullptr, clear_words, clear_count};
+    const PermuteExtras ex = {nullptr, clear_words, clear_count, nullptr};
     return permute_launch(x, x_dtype, expert_ids, expand_idx, row_off, 0, smooth, tokens, hidden, topk, experts, q,
                           single_window(q1, xs, experts, tokens * topk), st, ex);
 }

@@ -16,6 +16,7 @@
 
 #include "zbal_device.h"
 #include "zbal_hip_kernels.h"
+#include "zbal_layout_rank.h"
 
 #define ZB_MAX_EXPERTS 1024
 #define ZB_LAYOUT_THREADS 256
@@ -86,60 +87,6 @@ layout_hist_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int exper
     }
     __syncthreads();
     for (int e = threadIdx.x; e < experts; e += blockDim.x) scratch[(int64_t)blockIdx.x * experts + e] = hist[e];
-}
-
-/*
- * Stable ranks of the picks [p0, p1) of one block: `run[e]` holds the number of earlier picks of expert e on entry
- * and the number up to p1 on return. Picks are taken 64 per wave at a time; lanes holding the same expert find
- * each other by intersecting one ballot per index bit. The waves do not take turns: each leaves the size of its
- * groups in `cnt` (one byte per wave and expert, a group has at most 64 members) and a pick's rank is the running
- * count plus the groups of the waves before its own. Ends on a barrier.
- */
-template <typename IdxT>
-__device__ __forceinline__ void rank_picks(const IdxT *__restrict__ idx, int64_t p0, int64_t p1, int experts, int nbits,
-                                           int32_t *run, uint8_t *cnt /* [waves][experts rounded up to 4] */,
-                                           int32_t *__restrict__ send_token_idx)
-{
-    const int np = (int)(p1 - p0);
-    const int threads = blockDim.x, nwaves = threads >> 6;
-    const int iters = (np + threads - 1) / threads;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint64_t lt_mask = (lane == 0) ? 0ull : (~0ull >> (64 - lane));
-    const int pad = (experts + 3) & ~3;
-
-    for (int it = 0; it < iters; ++it) {
-        const int64_t i = p0 + (int64_t)it * threads + threadIdx.x;
-        int64_t e64 = (i < p1) ? (int64_t)idx[i] : -1;
-        for (int j = threadIdx.x; j < nwaves * pad / 4; j += threads) reinterpret_cast<uint32_t *>(cnt)[j] = 0u;
-        const bool valid = (e64 >= 0 && e64 < experts);
-        const int e = valid ? (int)e64 : 0;
-        uint64_t peers = __ballot(valid);
-        for (int bit = 0; bit < nbits; ++bit) {
-            const bool one = (e >> bit) & 1;
-            const uint64_t bal = __ballot(valid && one);
-            peers &= one ? bal : ~bal;
-        }
-        const int before = __popcll(peers & lt_mask);
-        const int group = __popcll(peers);
-        const bool last = valid && ((peers >> lane) >> 1) == 0; /* highest lane of its group */
-        __syncthreads();
-        if (last) cnt[wave * pad + e] = (uint8_t)group;
-        __syncthreads();
-        if (valid) {
-            int32_t basev = run[e];
-            for (int w = 0; w < wave; ++w) basev += cnt[w * pad + e];
-            send_token_idx[i] = basev + before;
-        } else if (i < p1) {
-            send_token_idx[i] = -1;
-        }
-        __syncthreads();
-        for (int e2 = threadIdx.x; e2 < experts; e2 += threads) {
-            int32_t sum = 0;
-            for (int w = 0; w < nwaves; ++w) sum += cnt[w * pad + e2];
-            run[e2] += sum;
-        }
-        __syncthreads();
-    }
 }
 
 template <typename IdxT>
@@ -288,6 +235,46 @@ layout_fused_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int expe
             if (nums_typed) nums_typed[e] = token_nums_type == 0 ? (int64_t)s : (int64_t)c;
         }
     }
+}
+
+/*
+ * The part of the layout that needs no other block: every block ranks the picks of its own token range among
+ * themselves (send_token_idx = position among the range's picks of the same expert) and leaves the range's histogram
+ * in hist[block][experts]. The permute kernel that follows turns the histograms into offsets on its own (dispatch.hip,
+ * table mode), so this launch is all there is in front of it: no counting of the ranges before, no scan.
+ */
+template <typename IdxT>
+__global__ void __launch_bounds__(ZB_FUSED_THREADS)
+layout_ranges_kernel(const IdxT *__restrict__ idx, int tokens, int topk, int experts, int tpb, int nbits,
+                     const uint8_t *__restrict__ active_mask, int32_t *__restrict__ send_token_idx,
+                     int32_t *__restrict__ hist)
+{
+    __shared__ int32_t run[ZB_MAX_EXPERTS];
+    __shared__ int32_t s_active;
+    __shared__ __align__(16) uint8_t cnt[ZB_FUSED_THREADS / 64 * ZB_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) run[e] = 0;
+    if (threadIdx.x == 0) s_active = 0;
+    __syncthreads();
+    int active = tokens;
+    if (active_mask) {          /* the first sum(mask) tokens are routed, the picks of the others get rank -2 (layout_fused_kernel) */
+        int part = 0;
+        for (int t = threadIdx.x; t < tokens; t += blockDim.x) part += active_mask[t] != 0;
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) part += __shfl_xor(part, off, 64);
+        if ((threadIdx.x & 63) == 0 && part) atomicAdd(&s_active, part);
+        __syncthreads();
+        active = s_active;
+    }
+    int tok0 = blockIdx.x * tpb;
+    int tok1 = tok0 + tpb;
+    if (tok1 > tokens) tok1 = tokens;
+    for (int64_t i = (int64_t)(tok0 > active ? tok0 : active) * topk + threadIdx.x; i < (int64_t)tok1 * topk; i += blockDim.x)
+        send_token_idx[i] = -2;
+    if (tok0 > active) tok0 = active;
+    if (tok1 > active) tok1 = active;
+    rank_picks(idx, (int64_t)tok0 * topk, (int64_t)tok1 * topk, experts, nbits, run, cnt, send_token_idx);
+    /* rank_picks ends on a barrier: run[] is the range's histogram */
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) hist[(int64_t)blockIdx.x * experts + e] = run[e];
 }
 
 /*
@@ -552,6 +539,17 @@ int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_
                                                                     p.tokens_per_block, ceil_log2(experts), token_nums_type,
                                                                     active_mask, send_token_idx, incl_i32, row_off,
                                                                     counts_i64, nums_typed);
+    return zbalhip_check_launch();
+}
+
+/* ranks within token ranges + one histogram per range, for the permute kernel's table mode; returns the ranges' size */
+int32_t zbalhip_layout_ranges_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
+                                       const uint8_t *active_mask, int32_t *send_token_idx, int32_t *hist, int nblk,
+                                       int tokens_per_block, hipStream_t st)
+{
+    layout_ranges_kernel<int32_t><<<nblk, ZB_FUSED_THREADS, 0, st>>>(idx, (int)tokens, (int)topk, (int)experts,
+                                                                    tokens_per_block, ceil_log2(experts), active_mask,
+                                                                    send_token_idx, hist);
     return zbalhip_check_launch();
 }
 
