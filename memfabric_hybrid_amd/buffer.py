@@ -315,22 +315,54 @@ class Buffer:
         p.zbal_prepacked = True
         return p
 
+    @staticmethod
+    def _weight_key(w: torch.Tensor):
+        return (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
+
+    def _cache_get(self, key, sources):
+        """The cached pre-packed form under `key`, or None. An entry is good only while every tensor it was made
+        from is alive: once one is freed the allocator may hand its address to other weights of the same shape, and
+        address, shape and version would still match."""
+        entry = self._packed.pop(key, None)
+        if entry is None or any(r() is None for r in entry[0]):
+            return None
+        self._packed[key] = entry        # most recently used last
+        return entry[1]
+
+    def _cache_put(self, key, sources, packed):
+        self._packed[key] = ([weakref.ref(t) for t in sources], packed)
+        while len(self._packed) > 16:    # a tensor list is one entry, however many experts it has
+            del self._packed[next(iter(self._packed))]
+        return packed
+
     def _packed_weight(self, w: torch.Tensor, int4: bool) -> torch.Tensor:
         if getattr(w, "zbal_prepacked", False):
             return w
-        # An entry is good only while the tensor it was made from is alive: once that tensor is freed the allocator may
-        # hand its address to other weights of the same shape, and address, shape and version would still match.
-        key = (w.data_ptr(), tuple(w.shape), w.dtype, w._version)
-        entry = self._packed.pop(key, None)
-        if entry is not None and entry[0]() is None:
-            entry = None
-        if entry is None:
+        key = self._weight_key(w)
+        packed = self._cache_get(key, [w])
+        if packed is None:
             w3 = w if w.dim() == 3 else w.unsqueeze(0)
-            entry = (weakref.ref(w), self.prepack_weight(w3.contiguous(), int4=int4))
-        self._packed[key] = entry        # most recently used last
-        while len(self._packed) > 16:
-            del self._packed[next(iter(self._packed))]
-        return entry[1]
+            packed = self._cache_put(key, [w], self.prepack_weight(w3.contiguous(), int4=int4))
+        return packed
+
+    def _packed_weight_list(self, ws, int4: bool):
+        """A list of per-expert weights -> the list of their pre-packed forms. The whole list is one cache entry and
+        one pre-pack launch (the experts stacked); the per-expert results are views of that one tensor."""
+        ws = list(ws)
+        if all(getattr(t, "zbal_prepacked", False) for t in ws):
+            return ws
+        key = ("list",) + tuple(self._weight_key(t) for t in ws)
+        packed = self._cache_get(key, ws)
+        if packed is None:
+            stacked = torch.stack([t if t.dim() == 2 else t.squeeze(0) for t in ws], 0)
+            whole = self.prepack_weight(stacked, int4=int4)
+            views = []
+            for e in range(len(ws)):
+                v = whole[e:e + 1]
+                v.zbal_prepacked = True
+                views.append(v)
+            packed = self._cache_put(key, ws, views)
+        return packed
 
     def topk_route(self, logits: torch.Tensor, num_topk: int, idx_dtype=torch.int64):
         """Extension: softmax + top-k router; returns (topk_idx, topk_weights)."""
@@ -361,8 +393,8 @@ class Buffer:
                   "Please pass share_gmm1_h_len with the correct value to avoid kernel errors.")
         int4 = quant_mode == 3
         if is_tensor_list:
-            w1 = [self._packed_weight(t, int4) for t in gmm1_permuted_weight]
-            w2 = [self._packed_weight(t, int4) for t in gmm2_weight]
+            w1 = self._packed_weight_list(gmm1_permuted_weight, int4)
+            w2 = self._packed_weight_list(gmm2_weight, int4)
         else:
             w1, w2 = self._packed_weight(gmm1_permuted_weight, int4), self._packed_weight(gmm2_weight, int4)
         sw1 = self._packed_weight(share_gmm1_weight, int4) if has_share else None

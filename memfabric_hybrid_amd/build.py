@@ -82,5 +82,31 @@ def build_library(force=False, verbose=False):
     return LIB
 
 
+def build_asan_library():
+    """The C++ host layer under AddressSanitizer and UndefinedBehaviorSanitizer (as the reference builds its unit
+    tests, CMakeLists.txt:73-80), linked with the library's ordinary kernel objects, into lib/libzbal_asan.so. For the
+    host-side tests on a machine without a GPU (the kernels are never launched there):
+
+        make -C oracle asan && python -m memfabric_hybrid_amd.build --asan
+        LD_PRELOAD=$(gcc -print-file-name=libasan.so) ASAN_OPTIONS=detect_leaks=0 \
+            ZBAL_LIB=memfabric_hybrid_amd/lib/libzbal_asan.so ZBAL_ORACLE_LIB=oracle/_build/libzbal_oracle_asan.so \
+            python -m pytest tests/test_capi_host.py tests/test_oracle_pins.py -q
+    """
+    build_library()
+    san = ["-fsanitize=address,undefined", "-fno-omit-frame-pointer", "-fno-sanitize-recover=undefined", "-g", "-O1"]
+    objs = [os.path.join(OBJ, k + ".o") for k in KERNELS]
+    for h in HOST:
+        obj = os.path.join(OBJ, h + ".asan.o")
+        _run(["g++"] + [f for f in HOST_FLAGS if f != "-O2"] + san + INCLUDES + ["-c", os.path.join(CSRC, "host", h + ".cpp"), "-o", obj])
+        objs.append(obj)
+    out = os.path.join(LIB_DIR, "libzbal_asan.so")
+    _run(["g++", "-shared", "-fPIC"] + san + ["-o", out] + objs + ["-L" + os.path.join(ROCM, "lib"), "-lamdhip64", "-lpthread",
+                                                                     "-Wl,-rpath," + os.path.join(ROCM, "lib")])
+    return out
+
+
 if __name__ == "__main__":
-    print(build_library(force="--force" in sys.argv, verbose=True))
+    if "--asan" in sys.argv:
+        print(build_asan_library())
+    else:
+        print(build_library(force="--force" in sys.argv, verbose=True))

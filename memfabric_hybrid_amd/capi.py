@@ -10,7 +10,8 @@ import ctypes
 import os
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_PKG, "lib", "libzbal.so")
+# ZBAL_LIB: another build of the library (the host layer under sanitizers, `python -m memfabric_hybrid_amd.build --asan`)
+LIB_PATH = os.environ.get("ZBAL_LIB") or os.path.join(_PKG, "lib", "libzbal.so")
 
 ZBAL_MAX_TENSOR_DIM = 12
 ZBAL_COMM_NAME_MAX = 128
@@ -186,7 +187,21 @@ CXX_SIGNATURES = {
     "ZBALOpDispatchLowLatency": [_TI, _TI, _i64, _i64, _i64, _i64, _i64, _i64, _i64, _TI, _TI, _TI, _TI, _TI, _TI, _TI, _vp,
                                  _GI, _i64],
     "ZBALOpCombineLowLatency": [_TI, _TI, _TI, _TI, _TI, _TI, _i64, _vp, _GI, _i64],
+    # ... isTensorList, tilingDevBuf, const std::string &groupName (see std_string), stream, ep group, tp group, flags, needTilingCopy
+    "ZBALOpFusedDeepMoe": [_TI] * 18 + [_i64] * 5 + [_bool, _vp, _vp, _vp, _GI, _GI, _i64, _bool],
 }
+
+
+def std_string(text=b""):
+    """A libstdc++ std::string (the 32-byte small-string form) holding up to 15 bytes, for the one launcher that
+    takes a `const std::string &`: pointer to the characters, length, then the in-object character buffer. Keep the
+    returned buffer alive for the call and pass ctypes.addressof(buffer)."""
+    assert len(text) <= 15
+    buf = ctypes.create_string_buffer(32)
+    ctypes.c_uint64.from_buffer(buf, 0).value = ctypes.addressof(buf) + 16
+    ctypes.c_uint64.from_buffer(buf, 8).value = len(text)
+    buf[16:16 + len(text)] = text
+    return buf
 _cxx = None
 
 

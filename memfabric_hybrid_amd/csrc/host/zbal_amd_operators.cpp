@@ -1,9 +1,13 @@
 /*
  * The reference's kernel-launcher functions (operators/npu/zbal_npu_operators.h:21-25, 47-97) on top of the HIP
- * backend: each builds the group description the backend works with from the CommGroupInfo it is handed and calls
- * the backend's operator, which checks the descriptors and launches the kernels. Nothing is kept between calls.
+ * backend: each finds (or, the first time a group is seen, builds) the backend object for the group the
+ * CommGroupInfo describes and calls the backend's operator, which checks the descriptors and launches the kernels.
  */
 #include "zbal_amd_operators.h"
+
+#include <cstring>
+#include <mutex>
+#include <vector>
 
 #include "zbal_hip_kernels.h"
 #include "zbal_host.h"
@@ -12,7 +16,21 @@ namespace {
 
 using namespace zbal;
 
-/* a communicator for one call; false (and a last error) when the group cannot be served */
+/*
+ * The backend objects built so far, by what identifies a group to the kernels: size, own rank, index, the distance
+ * between the ranks' memories and the world ranks of the members. A launch on a decode step must not pay for a new
+ * object (allocations, the one-time GEMM set-up) every time; a serving process sees a handful of groups.
+ */
+struct GroupKey {
+    uint16_t groupSize, myGroupRank;
+    uint32_t groupIndex;
+    uint64_t localDeviceMemSize;
+    uint16_t worldRank[ZBALHIP_MAX_REDUCE_PEERS];
+};
+std::mutex gGroupsMutex;
+std::vector<std::pair<GroupKey, CommunicatorPtr>> gGroups;
+
+/* the communicator of the group; false (and a last error) when the group cannot be served */
 bool GroupOf(const char *op, const CommGroupInfo &g, CommunicatorPtr *out)
 {
     ZBAL_VALIDATE_RETURN(g.groupSize >= 1 && g.groupSize <= ZBALHIP_MAX_REDUCE_PEERS,
@@ -20,6 +38,22 @@ bool GroupOf(const char *op, const CommGroupInfo &g, CommunicatorPtr *out)
     ZBAL_VALIDATE_RETURN(g.myGroupRank < g.groupSize, op << " failed as rank " << g.myGroupRank << " is not in the group", false);
     ZBAL_VALIDATE_RETURN(g.groupSize == 1 || g.localDeviceMemSize != 0,
                          op << " failed as localDeviceMemSize is 0 for a group of " << g.groupSize, false);
+    GroupKey key;
+    std::memset(&key, 0, sizeof(key));
+    key.groupSize = (uint16_t)g.groupSize;
+    key.myGroupRank = (uint16_t)g.myGroupRank;
+    key.groupIndex = (uint32_t)g.groupIndex;
+    if (g.groupSize > 1) {
+        key.localDeviceMemSize = g.localDeviceMemSize;
+        for (uint32_t r = 0; r < g.groupSize; ++r) key.worldRank[r] = (uint16_t)g.peerGroupRank2WorldRank[r];
+    }
+    std::lock_guard<std::mutex> guard(gGroupsMutex);
+    for (const auto &kv : gGroups) {
+        if (std::memcmp(&kv.first, &key, sizeof(key)) == 0) {
+            *out = kv.second;
+            return true;
+        }
+    }
     GroupInfo info;
     info.name = "kernel-seam";
     info.groupSize = g.groupSize;
@@ -32,6 +66,8 @@ bool GroupOf(const char *op, const CommGroupInfo &g, CommunicatorPtr *out)
         info.worldRank.assign(g.peerGroupRank2WorldRank, g.peerGroupRank2WorldRank + g.groupSize);
     }
     *out = MakeGpuCommunicator(info);
+    if (gGroups.size() >= 256) gGroups.clear(); /* a bound, not a policy: groups are few and long-lived */
+    gGroups.emplace_back(key, *out);
     return true;
 }
 
@@ -178,6 +214,11 @@ int32_t ZBALOpFusedDeepMoe(const zbal_tensor_info_t *x, const zbal_tensor_info_t
     const char *op = "FusedDeepMoe";
     ZB_NEED(op, x); ZB_NEED(op, expertIds); ZB_NEED(op, gmm1Weight); ZB_NEED(op, gmm1Scale); ZB_NEED(op, gmm2Weight);
     ZB_NEED(op, gmm2Scale); ZB_NEED(op, expertScales); ZB_NEED(op, output); ZB_NEED(op, expertTokenNums); ZB_NEED(op, workspace);
+    ZBAL_VALIDATE_RETURN(moeExpertNum > 0, op << " failed as moeExpertNum " << moeExpertNum << " is invalid", Z_INVALID_PARAM);
+    ZBAL_VALIDATE_RETURN(gmm1HLen > 0, op << " failed as gmm1HLen " << gmm1HLen << " is invalid", Z_INVALID_PARAM);
+    if (!SharedExpertArgsConsistent(op, shareGmm1Weight, shareGmm1Scale, shareGmm2Weight, shareGmm2Scale, shareSmoothScales,
+                                    shareOutput, shareGmm1HLen))
+        return Z_INVALID_PARAM;
     CommunicatorPtr c;
     if (!GroupOf(op, epGroupInfo, &c)) return Z_INVALID_PARAM;
     return c->FusedDeepMoe(x, expertIds, gmm1Weight, gmm1Scale, gmm2Weight, gmm2Scale, expertScales, expertSmoothScales,

@@ -47,6 +47,24 @@ CommunicatorPtr Resolve(const char *op, zbal_comm_t comm)
 
 } // namespace
 
+namespace zbal {
+bool SharedExpertArgsConsistent(const char *op, const zbal_tensor_info_t *shareGmm1Weight,
+                                const zbal_tensor_info_t *shareGmm1Scale, const zbal_tensor_info_t *shareGmm2Weight,
+                                const zbal_tensor_info_t *shareGmm2Scale, const zbal_tensor_info_t *shareSmoothScales,
+                                const zbal_tensor_info_t *shareOutput, int64_t shareGmm1HLen)
+{
+    auto present = [](const zbal_tensor_info_t *t) { return t != nullptr && t->data != nullptr; };
+    const bool shared = present(shareGmm1Weight);
+    ZBAL_VALIDATE_RETURN(shared == present(shareGmm1Scale) && shared == present(shareGmm2Weight) &&
+                             shared == present(shareGmm2Scale) && shared == present(shareOutput) &&
+                             shared == (shareGmm1HLen > 0) && (shared || !present(shareSmoothScales)),
+                         op << " failed as the shared expert needs both weights, both scales, shareOutput and "
+                               "shareGmm1HLen > 0, or none of them",
+                         false);
+    return true;
+}
+} // namespace zbal
+
 /* ---- lifecycle: reference zbal_operations.cpp:23-114 ------------------------ */
 
 ZBAL_API int32_t zbal_comm_create(zbal_comm_options_t *options, zbal_comm_t *comm)
@@ -299,9 +317,9 @@ ZBAL_API int32_t zbal_fused_deep_moe(
     if (!Present("FusedDeepMoe", {{"x", x}, {"expertIds", expertIds}, {"gmm1Weight", gmm1Weight}, {"gmm1Scale", gmm1Scale}, {"gmm2Weight", gmm2Weight}, {"gmm2Scale", gmm2Scale}, {"expertScales", expertScales}, {"output", output}, {"expertTokenNums", expertTokenNums}, {"workspace", workspace}})) return Z_INVALID_PARAM;
     ZBAL_VALIDATE_RETURN(moeExpertNum > 0, "FusedDeepMoe failed as moeExpertNum " << moeExpertNum << " is invalid", Z_INVALID_PARAM);
     ZBAL_VALIDATE_RETURN(gmm1HLen > 0, "FusedDeepMoe failed as gmm1HLen " << gmm1HLen << " is invalid", Z_INVALID_PARAM);
-    auto present = [](const zbal_tensor_info_t *t) { return t != nullptr && t->data != nullptr; };
-    const bool shared = present(shareGmm1Weight);
-    ZBAL_VALIDATE_RETURN(shared == present(shareGmm1Scale) && shared == present(shareGmm2Weight) && shared == present(shareGmm2Scale) && shared == present(shareOutput) && shared == (shareGmm1HLen > 0) && (shared || !present(shareSmoothScales)), "FusedDeepMoe failed as the shared expert needs both weights, both scales, shareOutput and shareGmm1HLen > 0, or none of them", Z_INVALID_PARAM);
+    if (!SharedExpertArgsConsistent("FusedDeepMoe", shareGmm1Weight, shareGmm1Scale, shareGmm2Weight, shareGmm2Scale,
+                                    shareSmoothScales, shareOutput, shareGmm1HLen))
+        return Z_INVALID_PARAM;
     CommunicatorPtr c = Resolve("FusedDeepMoe", comm);
     if (!c) return Z_INVALID_PARAM;
     return c->FusedDeepMoe(x, expertIds, gmm1Weight, gmm1Scale, gmm2Weight, gmm2Scale, expertScales, expertSmoothScales,

@@ -223,6 +223,15 @@ uint32_t Count();
 void DumpAllTraces();
 } // namespace registry
 
+/*
+ * The shared expert of the fused operator comes as a set: both weights, both scales, shareOutput and a positive
+ * shareGmm1HLen, or none of them (smooth scales only with it). One check for the C API and the launcher seam.
+ */
+bool SharedExpertArgsConsistent(const char *op, const zbal_tensor_info_t *shareGmm1Weight,
+                                const zbal_tensor_info_t *shareGmm1Scale, const zbal_tensor_info_t *shareGmm2Weight,
+                                const zbal_tensor_info_t *shareGmm2Scale, const zbal_tensor_info_t *shareSmoothScales,
+                                const zbal_tensor_info_t *shareOutput, int64_t shareGmm1HLen);
+
 /* Layout of the fused operator's workspace; one function so that sizing and carving cannot diverge. */
 struct FusedWorkspace {
     uint64_t q1, xs, expand_idx, counts, row_off, layout_scratch, q2, scale2, sgl, y, total;

@@ -6,9 +6,13 @@
  * and no symmetric heap, peers being windows registered per communicator.
  */
 #include <atomic>
+#include <cerrno>
 #include <csignal>
 #include <cstdio>
 #include <cstring>
+#include <thread>
+
+#include <semaphore.h>
 
 #include <hip/hip_runtime.h>
 
@@ -54,11 +58,69 @@ BootState &Boot()
 
 using namespace zbal;
 
-/* SIGUSR1 writes every communicator's device trace, as in the reference (common/zbal_signal_handler.cpp:21-29) */
-static void DumpTracesOnSignal(int sig)
+/*
+ * SIGUSR1 asks for every communicator's device trace, as in the reference (common/zbal_signal_handler.cpp:21-29).
+ * Writing the traces takes the registry's lock, synchronises the device, allocates and writes files: nothing a
+ * signal handler may do (the signal can land on a thread that holds that very lock). The handler only posts a
+ * semaphore and passes the signal on to the handler that was installed before bootstrap; a helper thread, started by
+ * bootstrap and joined by unbootstrap, waits on the semaphore and writes the traces from ordinary code -- also when
+ * every other thread of the process is stuck, which is when one wants them.
+ */
+namespace {
+sem_t gDumpRequests;
+std::atomic<bool> gDumpThreadStop{false};
+std::thread gDumpThread;
+struct sigaction gPreviousUsr1;
+bool gHandlerInstalled = false;
+
+void OnUsr1(int sig, siginfo_t *info, void *context)
 {
-    if (sig == SIGUSR1) registry::DumpAllTraces();
+    const int saved = errno;
+    sem_post(&gDumpRequests);
+    errno = saved;
+    if (gPreviousUsr1.sa_flags & SA_SIGINFO) {
+        if (gPreviousUsr1.sa_sigaction != nullptr) gPreviousUsr1.sa_sigaction(sig, info, context);
+    } else if (gPreviousUsr1.sa_handler != SIG_DFL && gPreviousUsr1.sa_handler != SIG_IGN && gPreviousUsr1.sa_handler != nullptr) {
+        gPreviousUsr1.sa_handler(sig);
+    }
 }
+
+void DumpThreadMain()
+{
+    for (;;) {
+        while (sem_wait(&gDumpRequests) != 0 && errno == EINTR) {}
+        if (gDumpThreadStop.load(std::memory_order_acquire)) return;
+        registry::DumpAllTraces();
+    }
+}
+
+void InstallUsr1()
+{
+    sem_init(&gDumpRequests, 0, 0);
+    gDumpThreadStop.store(false, std::memory_order_release);
+    gDumpThread = std::thread(DumpThreadMain);
+    struct sigaction act;
+    std::memset(&act, 0, sizeof(act));
+    act.sa_sigaction = OnUsr1;
+    act.sa_flags = SA_SIGINFO | SA_RESTART;
+    sigemptyset(&act.sa_mask);
+    gHandlerInstalled = sigaction(SIGUSR1, &act, &gPreviousUsr1) == 0;
+}
+
+void RemoveUsr1()
+{
+    if (gHandlerInstalled) { /* the process gets back the SIGUSR1 handler it had before bootstrap */
+        sigaction(SIGUSR1, &gPreviousUsr1, nullptr);
+        gHandlerInstalled = false;
+    }
+    if (gDumpThread.joinable()) {
+        gDumpThreadStop.store(true, std::memory_order_release);
+        sem_post(&gDumpRequests);
+        gDumpThread.join();
+        sem_destroy(&gDumpRequests);
+    }
+}
+} // namespace
 
 /* the kernel launchers' way to leave a last-error text (declared in kernels/zbal_device.h) */
 void zbalhip_set_last_error(const char *text) { ZBAL_LOG_AND_SET_LAST_ERROR(text); }
@@ -128,7 +190,7 @@ __attribute__((visibility("default"))) int32_t zbal_bootstrap(zbal_bootstrap_opt
         ZBAL_VALIDATE_RETURN(e == hipSuccess, "Bootstrap failed as hipSetDevice failed: " << hipGetErrorString(e),
                              Z_INIT_BOOTSTRAP_FAILED);
     }
-    std::signal(SIGUSR1, DumpTracesOnSignal); /* installed by bootstrap, reference bootstrap/zbal_bootstrap_default.cpp:102 */
+    InstallUsr1(); /* installed by bootstrap, reference bootstrap/zbal_bootstrap_default.cpp:102 */
     st.bootstrapped = true;
     st.worldSize = options->worldSize;
     st.rankId = options->rankId;
@@ -149,6 +211,7 @@ __attribute__((visibility("default"))) int32_t zbal_unbootstrap(uint32_t flags)
     std::lock_guard<std::mutex> guard(gBootMutex);
     BootState &st = Boot();
     ZBAL_VALIDATE_RETURN(st.bootstrapped, "Unbootstrap failed as not bootstrapped", Z_CANNOT_UNBOOTSTRAP);
+    RemoveUsr1(); /* before the communicators go: the helper thread must not be writing their traces */
     registry::DestroyAll();
     st = BootState();
     return Z_OK;

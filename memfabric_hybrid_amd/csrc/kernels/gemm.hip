@@ -30,6 +30,7 @@
  * the workgroups resident on an XCD share both their A and their W slabs in
  * that XCD's L2.
  */
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 
@@ -1168,6 +1169,11 @@ extern "C" int32_t zbalhip_gmm2_dequant(const void *a, const float *a_scale, con
 
 extern "C" int32_t zbalhip_gemm_prepare(void)
 {
+    /* once per device and process: later calls (every communicator that is created makes one) cost one device query */
+    static std::atomic<bool> prepared[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return ZBALHIP_RT_ERROR;
+    if (prepared[dev].load(std::memory_order_acquire)) return ZBALHIP_OK;
     int32_t rc = prepare_mode<MODE_W8A8, true, ZDT_BF16>();
     if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_FP8, true, ZDT_BF16>();
     if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W4A8, true, ZDT_BF16>();
@@ -1177,5 +1183,6 @@ extern "C" int32_t zbalhip_gemm_prepare(void)
     if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_FP8, false, ZDT_FP16>();
     if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W4A8, false, ZDT_BF16>();
     if (rc == ZBALHIP_OK) rc = prepare_mode<MODE_W4A8, false, ZDT_FP16>();
+    if (rc == ZBALHIP_OK) prepared[dev].store(true, std::memory_order_release);
     return rc;
 }

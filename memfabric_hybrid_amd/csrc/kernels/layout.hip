@@ -34,18 +34,30 @@ namespace {
 
 constexpr int ZB_MAX_DEVICES = 64;
 
-/* device address of this GPU's copy of `scratch`, looked up on the first call with that GPU current */
-int32_t *static_scratch_of(int dev)
+/*
+ * This GPU's copy of `scratch`: its device address, looked up on the first call with that GPU current, and an event
+ * that marks the end of the last launch sequence that used it. Calls are issued under `mu`, each waiting for that
+ * event on its own stream first and recording it again after its last launch, so two callers on different streams
+ * (or threads) take turns on the array instead of racing on it.
+ */
+struct StaticScratch {
+    std::mutex mu;
+    int32_t *addr = nullptr;
+    hipEvent_t last_use = nullptr;
+};
+
+StaticScratch *static_scratch_of(int dev)
 {
-    static std::mutex mu;
-    static int32_t *addr[ZB_MAX_DEVICES] = {};
-    std::lock_guard<std::mutex> guard(mu);
-    if (addr[dev] == nullptr) {
+    static StaticScratch per_device[ZB_MAX_DEVICES];
+    StaticScratch &s = per_device[dev];
+    std::lock_guard<std::mutex> guard(s.mu);
+    if (s.addr == nullptr) {
         void *p = nullptr;
         if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || p == nullptr) return nullptr;
-        addr[dev] = static_cast<int32_t *>(p);
+        if (hipEventCreateWithFlags(&s.last_use, hipEventDisableTiming) != hipSuccess) return nullptr;
+        s.addr = static_cast<int32_t *>(p);
     }
-    return addr[dev];
+    return &s;
 }
 
 struct LayoutPlan {
@@ -627,15 +639,26 @@ extern "C" int32_t zbalhip_dispatch_layout_static(const void *topk_idx, int32_t 
         return ZBALHIP_INVALID;
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= ZB_MAX_DEVICES) return ZBALHIP_RT_ERROR;
-    int32_t *hist = static_scratch_of(dev);
-    if (hist == nullptr) return ZBALHIP_RT_ERROR;
+    StaticScratch *ss = static_scratch_of(dev);
+    if (ss == nullptr) return ZBALHIP_RT_ERROR;
+    hipStream_t st = (hipStream_t)stream;
+    /*
+     * Under stream capture the order of the array's users is the captured graph's own business (an event recorded
+     * outside of the capture cannot be waited for inside it); everywhere else this call queues behind the last one.
+     */
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    const bool capturing = st != nullptr && hipStreamIsCapturing(st, &capture) == hipSuccess && capture != hipStreamCaptureStatusNone;
+    std::lock_guard<std::mutex> guard(ss->mu);
+    if (!capturing && hipStreamWaitEvent(st, ss->last_use, 0) != hipSuccess) return ZBALHIP_RT_ERROR;
     /* the histogram kernel writes every row that the rank and scan kernels read: nothing has to start at zero */
     int nblk = 0;
     int32_t rc = zbalhip_layout_internal(topk_idx, idx_is_i64, tokens, experts, topk, ranks, tokens_per_rank,
-                                         send_token_idx, hist, ZBALHIP_LAYOUT_MAX_BLOCKS, &nblk, (hipStream_t)stream);
-    if (rc != ZBALHIP_OK) return rc;
-    return zbalhip_scan_internal(hist, nblk, experts, topk, 1, tokens_per_expert, nullptr, nullptr, nullptr, nullptr,
-                                 nullptr, nullptr, nullptr, (hipStream_t)stream);
+                                         send_token_idx, ss->addr, ZBALHIP_LAYOUT_MAX_BLOCKS, &nblk, st);
+    if (rc == ZBALHIP_OK)
+        rc = zbalhip_scan_internal(ss->addr, nblk, experts, topk, 1, tokens_per_expert, nullptr, nullptr, nullptr, nullptr,
+                                   nullptr, nullptr, nullptr, st);
+    if (!capturing && hipEventRecord(ss->last_use, st) != hipSuccess && rc == ZBALHIP_OK) rc = ZBALHIP_RT_ERROR;
+    return rc;
 }
 
 extern "C" int32_t zbalhip_dispatch_notify(const int32_t *const *tokens_per_expert, int32_t ranks, int32_t my_rank,

@@ -11,7 +11,8 @@ import subprocess
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(_HERE, "_build", "libzbal_oracle.so")
+# ZBAL_ORACLE_LIB: another build of the same source (the sanitizer build, `make -C oracle asan`)
+_LIB_PATH = os.environ.get("ZBAL_ORACLE_LIB") or os.path.join(_HERE, "_build", "libzbal_oracle.so")
 
 DT_INT8, DT_INT16, DT_INT32, DT_INT64 = 0, 1, 2, 3
 DT_FP16, DT_FP32, DT_BF16 = 6, 7, 8

@@ -207,6 +207,50 @@ def test_fused_workspace_size_is_monotonic(lib):
     assert f(128, 7168, 8, 32, 4096, 100, 0) == 0
 
 
+def reference_workspace_bytes(bs, h, gmm1_h_len, share_gmm1_h_len, experts_per_rank, ranks, topk, global_bs, aic_num):
+    """The size the reference's adaptor allocates for the fused operator's workspace, restated from
+    zbal_deepep.cpp:42-84 (ComputeWorkspaceSize; the host launcher checks against the same sum,
+    host/fused_deep_moe/zbal_kernel_fused_deep_moe_host.cpp:59-132): 16 MiB for the system plus regions each rounded
+    up to 512 bytes."""
+    up = lambda x: (x + 511) // 512 * 512
+    max_bs = global_bs // ranks
+    max_tokens = max_bs * ranks * min(topk, experts_per_rank)
+    gmm2_h, share_gmm2_h = gmm1_h_len // 2, share_gmm1_h_len // 2
+    share_tokens = bs if share_gmm1_h_len > 0 else 0
+    handled = max_tokens + share_tokens
+    x1 = up(handled * h)
+    x2 = up(max_tokens * gmm2_h + share_tokens * share_gmm2_h)
+    token_scale = up(handled * 4)
+    cv_swap = up(aic_num * 32 * 1024 * 4 * 4)
+    swiglu = (max_tokens * gmm1_h_len + share_tokens * share_gmm1_h_len) * 4
+    gmm2_out = max_tokens * h * 2
+    group_list = up(experts_per_rank * 8)
+    expand_idx = up(bs * topk * 4)
+    send_count = up(ranks * experts_per_rank * 4)
+    reserved = up(256 * 1024)
+    quant_ws = up(bs * topk * up(h + 4))
+    combine_ws = up(experts_per_rank * ranks * max_bs * h * 2)
+    return (16 << 20) + max(x1, x2) + token_scale + cv_swap + up(max(swiglu, gmm2_out)) + group_list + expand_idx + \
+        send_count + reserved + quant_ws + combine_ws
+
+
+@pytest.mark.parametrize("tokens,hidden,topk,experts,n1", [(256, 1024, 2, 8, 2048),        # the small CPU-reference layer
+                                                           (4096, 7168, 8, 32, 4096),      # prefill share
+                                                           (128, 7168, 8, 32, 4096),       # decode share
+                                                           (16384, 4096, 8, 128, 3072),    # W4A8 layer
+                                                           (1, 7168, 8, 256, 4096), (0, 7168, 8, 32, 4096)])
+def test_a_workspace_sized_by_the_reference_is_large_enough(lib, tokens, hidden, topk, experts, n1):
+    """A caller that keeps the reference adaptor's own sizing (one rank, global_bs = bs as the adaptor defaults it)
+    hands zbal_fused_deep_moe at least what this build asks for: every quant mode, with and without a shared expert.
+    The cube-core count enters the reference's sum through a 512 KiB-per-core swap area; the smallest count of any
+    Ascend part (20) gives the smallest reference size."""
+    for share_n1 in (0, n1):
+        want = reference_workspace_bytes(max(tokens, 1), hidden, n1, share_n1, experts, 1, topk, max(tokens, 1), aic_num=20)
+        for quant_mode in (0, 1, 2, 3):
+            ours = lib.zbal_fused_deep_moe_workspace_size(tokens, hidden, topk, experts, n1, share_n1, quant_mode)
+            assert 0 < ours <= want, (share_n1, quant_mode, ours, want)
+
+
 def test_kernel_seam_types_and_exports():
     """CommGroupInfo keeps the reference's layout (zbal_comm_host_device_struct.h:133-151: 2160 bytes,
     peerGroupRank2WorldRank at 64) and the nine launcher functions of zbal_npu_operators.h are exported with C++
@@ -222,6 +266,52 @@ def test_kernel_seam_types_and_exports():
                      "ZBALOpDispatchNormal", "ZBALOpCombineNormal", "ZBALOpDispatchLowLatency", "ZBALOpCombineLowLatency",
                      "ZBALOpFusedDeepMoe"}
     assert set(capi.CXX_SIGNATURES) <= names
+
+
+def test_launcher_seam_refuses_an_incomplete_shared_expert(lib):
+    """ZBALOpFusedDeepMoe with shared-expert weights but no shareOutput (or no scales) is refused with
+    Z_INVALID_PARAM like zbal_fused_deep_moe, before any descriptor is read or a device is touched."""
+    fn = capi.load_cxx()["ZBALOpFusedDeepMoe"]
+    byte = ctypes.c_char()
+    t = capi.TensorInfo()
+    t.data = ctypes.addressof(byte)
+    r, null = ctypes.byref(t), None
+    g = capi.CommGroupInfo()
+    g.groupSize, g.myGroupRank = 1, 0
+    name = capi.std_string(b"ep")
+
+    def call(share_w1, share_s1, share_w2, share_s2, share_out, share_n1):
+        return fn(r, r, r, r, r, r, r, null, share_w1, share_s1, share_w2, share_s2, null, null, r, share_out, r, r,
+                  8, 0, 0, 256, share_n1, False, None, ctypes.addressof(name), None, ctypes.byref(g), ctypes.byref(g), 0, True)
+    assert call(r, r, r, r, null, 256) == capi.Z_INVALID_PARAM
+    assert b"shared expert" in lib.zbal_get_last_error_msg()
+    assert call(r, null, r, r, r, 256) == capi.Z_INVALID_PARAM
+    assert call(r, r, r, r, r, 0) == capi.Z_INVALID_PARAM
+    assert call(null, null, null, null, r, 0) == capi.Z_INVALID_PARAM
+
+
+def test_sigusr1_is_deferred_chained_and_restored(lib):
+    """Bootstrap installs a SIGUSR1 handler that only wakes a helper thread (which writes the traces), passes the
+    signal on to the handler that was there before, and unbootstrap puts that one back and joins the thread."""
+    import signal
+    seen = []
+    before = signal.signal(signal.SIGUSR1, lambda *_: seen.append(1))
+    try:
+        opts = capi.BootstrapOptions()
+        assert lib.zbal_bootstrap_options_init(ctypes.byref(opts)) == 0
+        opts.flags = 1
+        assert lib.zbal_bootstrap(ctypes.byref(opts), None) == 0
+        rc, comm = make_comm(lib, b"sig_world", 1, 1, 0)
+        assert rc == 0
+        os.kill(os.getpid(), signal.SIGUSR1)
+        assert seen == [1]                                         # chained to the handler installed before bootstrap
+        assert lib.zbal_comm_dump_profiling_trace(comm) == 0       # the library stays usable while the helper thread works
+        assert lib.zbal_comm_destroy(comm, 0) == 0
+        assert lib.zbal_unbootstrap(0) == 0
+        os.kill(os.getpid(), signal.SIGUSR1)
+        assert seen == [1, 1]                                      # the old handler is back in place
+    finally:
+        signal.signal(signal.SIGUSR1, before)
 
 
 def test_deepep_buffer_signatures_follow_the_reference():

@@ -240,3 +240,29 @@ def test_fused_deep_moe_repacks_new_weights_at_a_reused_address(buffer):
         del g1_w, g2_w, out
     if len(seen) == 3:            # the allocator never handed an address out again: results were right, but the case went untested
         pytest.skip("the allocator did not re-use an address; the stale-cache case was not exercised")
+
+
+def test_fused_deep_moe_with_tensor_lists_packs_once(buffer, monkeypatch):
+    """Per-expert weight lists through Buffer.fused_deep_moe (32 experts, 64 weight tensors in all): bit-exact against
+    the oracle, the whole list pre-packed by one launch per operand, and a second call with the same tensors pre-packs
+    nothing."""
+    bs, hidden, ffn, num_experts, num_topk = 64, 256, 256, 32, 4
+    torch.manual_seed(11)
+    x = (torch.rand((bs, hidden), device="cuda") * 10 - 5).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(num_experts, device="cuda")[:num_topk] for _ in range(bs)]).to(torch.int32)
+    es = torch.rand((bs, num_topk), dtype=torch.float32, device="cuda")
+    g1 = [torch.randint(-16, 16, (hidden, ffn), dtype=torch.int8, device="cuda") for _ in range(num_experts)]
+    g2 = [torch.randint(-16, 16, (ffn // 2, hidden), dtype=torch.int8, device="cuda") for _ in range(num_experts)]
+    s1 = [(torch.rand(ffn, dtype=torch.float32, device="cuda") * 0.003 + 0.0015) for _ in range(num_experts)]
+    s2 = [(torch.rand(hidden, dtype=torch.float32, device="cuda") * 0.003 + 0.0015).to(torch.bfloat16) for _ in range(num_experts)]
+    packs = []
+    real = buffer.runtime.prepack_weight
+    monkeypatch.setattr(buffer.runtime, "prepack_weight", lambda w, int4=False: (packs.append(tuple(w.shape)), real(w, int4=int4))[1])
+    ref, counts = zo.fused_moe(host(x), zo.DT_BF16, host(ids), host(es), host(torch.stack(g1)), host(torch.stack(s1)),
+                               host(torch.stack(g2)), host(torch.stack(s2)), num_experts, 0)
+    for call in range(2):
+        out, nums = buffer.fused_deep_moe(x=x, topk_idx=ids, gmm1_permuted_weight=g1, gmm1_permuted_weight_scale=s1,
+                                          gmm2_weight=g2, gmm2_weight_scale=s2, topk_weights=es, num_experts=num_experts,
+                                          is_tensor_list=True)
+        assert np.array_equal(host(nums), counts) and np.array_equal(host(out), ref), call
+        assert packs == [(num_experts, hidden, ffn), (num_experts, ffn // 2, hidden)], (call, packs)

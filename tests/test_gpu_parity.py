@@ -424,6 +424,11 @@ def test_device_trace_ring_and_trace_viewer_dump(buf, tmp_path, monkeypatch):
         for f in files:
             os.remove(f)
         os.kill(os.getpid(), signal.SIGUSR1)
+        import time                                       # the handler only wakes the library's helper thread, which writes
+        deadline = time.time() + 10
+        while not glob.glob(str(tmp_path / "trace_view_1_*.json")) and time.time() < deadline:
+            time.sleep(0.02)
+        time.sleep(0.2)                                   # let it finish the file
         assert len(glob.glob(str(tmp_path / "trace_view_1_*.json"))) == 1
         # a second traced communicator has a ring of its own: destroying it leaves this one's tracing on
         other = create_group("traced_other", 1, 0)

@@ -340,3 +340,56 @@ def test_empty_batch_fused_and_low_latency(buf):
     assert rc == 0, capi.last_error()
     torch.cuda.synchronize()
     assert bool((nums == 0).all()) and bool((counts == 0).all())
+
+
+def test_fused_and_all_reduce_through_the_launcher_seam(buf):
+    """ZBALOpFusedDeepMoe and ZBALOpAllReduce, called the way the reference's communicator layer calls them (a
+    CommGroupInfo, a std::string group name), give the outer ABI's results bit for bit; a second call on the same
+    group reuses the backend object built by the first."""
+    lib, fn = buf.lib, capi.load_cxx()
+    ti, ref, st = capi.tensor_info, ctypes.byref, capi.stream_ptr()
+    T, H, K, E, I = 96, 512, 4, 8, 256
+    x = torch.from_numpy(bf16_normal((T, H), 1)).view(torch.int16).view(torch.bfloat16).cuda()
+    ids = torch.from_numpy(rng(2).integers(0, E, size=(T, K)).astype(np.int32)).cuda()
+    es = torch.from_numpy(rng(3).uniform(0, 1, (T, K)).astype(np.float32)).cuda()
+    w1 = buf.prepack_weight(torch.from_numpy(rng(4).integers(-16, 16, (E, H, 2 * I)).astype(np.int8)).cuda())
+    s1 = torch.from_numpy(rng(5).uniform(0.0015, 0.0045, (E, 2 * I)).astype(np.float32)).cuda()
+    w2 = buf.prepack_weight(torch.from_numpy(rng(6).integers(-16, 16, (E, I, H)).astype(np.int8)).cuda())
+    s2 = torch.from_numpy(rng(7).uniform(0.0015, 0.0045, (E, H)).astype(np.float32)).cuda().to(torch.bfloat16)
+    want, _, want_nums = buf.fused_deep_moe(x, ids, w1, s1, w2, s2, es, E, quant_mode=0)
+    ws = torch.empty(buf.fused_workspace_bytes(T, H, K, E, 2 * I, 0), dtype=torch.uint8, device="cuda")
+    g = capi.CommGroupInfo()
+    g.groupSize, g.myGroupRank = 1, 0
+    name = capi.std_string(b"ep_group")
+    null = ref(capi.TensorInfo())
+    pre = capi.WEIGHT_FORMAT_PREPACKED
+    for _ in range(2):
+        out = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+        nums = torch.zeros(E, dtype=torch.int64, device="cuda")
+        rc = fn["ZBALOpFusedDeepMoe"](ref(ti(x)), ref(ti(ids)), ref(ti(w1, weight_format=pre)), ref(ti(s1)),
+                                      ref(ti(w2, weight_format=pre)), ref(ti(s2)), ref(ti(es)), null, null, null, null, null,
+                                      null, null, ref(ti(out)), null, ref(ti(nums)), ref(ti(ws)), E, 0, 0, 2 * I, 0, False,
+                                      None, ctypes.addressof(name), st, ref(g), ref(g), 0, True)
+        assert rc == 0, capi.last_error()
+        assert torch.equal(out, want) and torch.equal(nums, want_nums)
+
+    # all-reduce over four windows that lie localDeviceMemSize bytes apart
+    R, n = 4, 3000
+    stride = (n * 4 + 255) // 256 * 256
+    whole = torch.zeros(R * stride, dtype=torch.uint8, device="cuda")
+    parts = [whole[r * stride:r * stride + n * 4].view(torch.float32) for r in range(R)]
+    for r in range(R):
+        parts[r].copy_(torch.from_numpy(rng(20 + r).standard_normal(n).astype(np.float32)))
+    ref_sum = parts[0].clone()
+    for r in range(1, R):
+        ref_sum = ref_sum + parts[r]
+    for me in range(R):
+        gi = capi.CommGroupInfo()
+        gi.groupSize, gi.myGroupRank, gi.localDeviceMemSize = R, me, stride
+        for i in range(R):
+            gi.peerGroupRank2WorldRank[i] = i
+        out = torch.zeros(n, dtype=torch.float32, device="cuda")
+        rc = fn["ZBALOpAllReduce"](parts[me].data_ptr(), out.data_ptr(), None, n, capi.DT_FP32, st, capi.REDUCE_SUM, ref(gi))
+        assert rc == 0, capi.last_error()
+        assert torch.equal(out, ref_sum)
+        assert gi.waitSymbol == 1

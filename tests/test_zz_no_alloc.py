@@ -60,3 +60,32 @@ def test_static_layout_refuses_what_the_scratch_cannot_hold():
                                             out.data_ptr(), None)
     assert rc == -2
     assert b"static scratch" in lib.zbal_get_last_error_msg()
+
+
+def test_static_layout_calls_on_two_streams_take_turns():
+    """Calls issued back to back on two streams share the one static scratch: the library queues each behind the
+    one before (an event per GPU), so both give the caller-scratch results although their streams are not ordered."""
+    lib = capi.load()
+    torch.cuda.set_device(0)
+    cases = []
+    for T, K, E, R, seed in ((5000, 8, 200, 4, 21), (4800, 8, 64, 2, 22), (5200, 6, 256, 8, 23), (300, 4, 16, 1, 24)):
+        idx = rng(seed).integers(-1, E + 1, size=(T, K)).astype(np.int32)
+        d_idx = torch.from_numpy(idx).cuda()
+        scratch = torch.empty((MAX_BLOCKS * E,), dtype=torch.int32, device="cuda")
+        want = [torch.empty(R, dtype=torch.int32, device="cuda"), torch.empty(E, dtype=torch.int32, device="cuda"),
+                torch.empty((T, K), dtype=torch.int32, device="cuda")]
+        assert lib.zbalhip_dispatch_layout(d_idx.data_ptr(), 0, T, E, K, R, want[0].data_ptr(), want[1].data_ptr(),
+                                           want[2].data_ptr(), scratch.data_ptr(), None) == 0
+        got = [torch.full_like(w, -7) for w in want]
+        cases.append((d_idx, T, K, E, R, want, got))
+    torch.cuda.synchronize()
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    for rep in range(3):
+        for i, (d_idx, T, K, E, R, want, got) in enumerate(cases):
+            st = streams[i % 2]
+            assert lib.zbalhip_dispatch_layout_static(d_idx.data_ptr(), 0, T, E, K, R, got[0].data_ptr(), got[1].data_ptr(),
+                                                      got[2].data_ptr(), st.cuda_stream) == 0
+    torch.cuda.synchronize()
+    for _, _, _, _, _, want, got in cases:
+        for w, g in zip(want, got):
+            assert torch.equal(w, g)
