@@ -117,8 +117,10 @@ ZBALHIP_API int32_t zbalhip_dispatch_normal(const void *x, int32_t x_dtype, cons
  * of `ranks` device pointers (the windows the rows were dispatched to, y_rows
  * rows each; a row past that is skipped); the row of a pick of expert e is
  * row base[e * ranks + my_rank] + send_token_idx of window e / (experts /
- * ranks). base_is_inclusive = 1 (ranks == 1 only) reads `base` as the
- * low-latency kernels' inclusive running counts (combine_low_latency.h:504-506).
+ * ranks). base_is_inclusive = 1 reads `base` as the low-latency kernels'
+ * inclusive running counts (combine_low_latency.h:504-506): the rows of index
+ * i = e * ranks + my_rank start at base[i - 1], at 0 where i is a multiple
+ * of `experts` (every rank's block of counts starts anew).
  */
 ZBALHIP_API int32_t zbalhip_combine(const void *const *y, int32_t ranks, int32_t my_rank, int64_t y_rows, int32_t dtype,
                         const int32_t *base, int32_t base_is_inclusive, const float *w, const int32_t *topk_idx,
@@ -140,6 +142,31 @@ ZBALHIP_API int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype,
                                      int32_t token_nums_type, void *expand_x, float *dynamic_scales,
                                      int32_t *expand_idx, int64_t *expert_token_nums, int32_t *ep_recv_counts,
                                      int32_t *scratch, int32_t scratch_blocks, void *stream);
+
+/*
+ * The same for a group of `ranks` modelled ranks (kernel
+ * dispatch_low_latency.h: counts of all ranks :344-345, 641-713, rows sent to
+ * the rank that owns the expert :760-844). expert_ids, expand_x and
+ * dynamic_scales are HOST arrays of `ranks` device pointers: every rank's
+ * [tokens, topk] ids (the reference's ranks push their counts to each other
+ * and wait; here the other ranks' ids are read where they lie, all ranks
+ * with the same tokens and topk) and every rank's receive window (dest_rows
+ * rows each; a row past that is dropped). all_counts [ranks * experts] =
+ * picks of expert e by rank s at s * experts + e (the reference's putOffset
+ * operand); ep_recv_counts [ranks * experts] = inclusive running sums at
+ * r * experts + le * ranks + s, starting anew for every destination rank r;
+ * expert_token_nums [experts / ranks] = what this rank receives per local
+ * expert (type 1) or the running sum (type 0); expand_idx [tokens, topk] =
+ * rank of each of this rank's picks among its own earlier picks of the same
+ * expert. A pick of expert e lands in window e / (experts / ranks) at row
+ * start(e * ranks + my_rank) + expand_idx.
+ */
+ZBALHIP_API int32_t zbalhip_dispatch_low_latency_ranks(const void *x, int32_t x_dtype, const int32_t *const *expert_ids,
+                                           int64_t tokens, int64_t hidden, int64_t topk, int64_t experts,
+                                           int32_t quant_mode, int32_t token_nums_type, void *const *expand_x,
+                                           float *const *dynamic_scales, int32_t ranks, int32_t my_rank,
+                                           int64_t dest_rows, int32_t *expand_idx, int64_t *expert_token_nums,
+                                           int32_t *ep_recv_counts, int32_t *all_counts, void *stream);
 
 /*
  * Device trace ring (reference aicore/common/zbal_kernel_trace.h:22-62, layout

@@ -145,6 +145,8 @@ SIGNATURES = {
     "zbalhip_fill_i32": (_i32, [_vp, _i64, _i32, _vp]),
     "zbalhip_fused_permute_quant": (_i32, [_vp, _i32, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp, _vp,
                                            _vp, _i64, _vp, _i32, _vp]),
+    "zbalhip_dispatch_low_latency_ranks": (_i32, [_vp, _i32, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _i32, _i32, _i64,
+                                                  _vp, _vp, _vp, _vp, _vp]),
     "zbalhip_gmm1_swiglu_quant": (_i32, [_vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _i64, _i32, _vp, _vp, _vp, _vp]),
     "zbalhip_gmm2_dequant": (_i32, [_vp, _vp, _vp, _vp, _i32, _vp, _i64, _i64, _i64, _i64, _i32, _i32, _vp, _vp]),
     "zbalhip_gemm_prepare": (_i32, []),

@@ -444,7 +444,9 @@ public:
                                int64_t) override
     {
         const char *op = "DispatchLowlatency";
-        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        const int64_t R = info_.groupSize, me = info_.myGroupRank;
+        ZBAL_VALIDATE_RETURN(R <= ZBALHIP_MAX_REDUCE_PEERS && moeExpertNum % R == 0,
+                             op << " failed as " << moeExpertNum << " experts do not split over a group of " << R, Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(sharedExpertRankNum == 0, op << " failed as shared expert ranks are not supported", Z_INVALID_PARAM);
         ZBAL_VALIDATE_RETURN(expertTokenNumsType == 0 || expertTokenNumsType == 1,
                              op << " failed as expertTokenNumsType " << expertTokenNumsType << " is invalid", Z_INVALID_PARAM);
@@ -460,9 +462,10 @@ public:
         ZBAL_VALIDATE_RETURN(rowBytes % 32 == 0, op << " failed as a row of " << rowBytes << " bytes is not a multiple of 32",
                              Z_INVALID_PARAM);
         const int64_t E = moeExpertNum;
-        ZB_CHECK(op, "expertTokenNumsOut", expertTokenNumsOut, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E);
-        ZB_CHECK(op, "epRecvCountsOut", epRecvCountsOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
-        ZB_CHECK(op, "putOffset", putOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E);
+        /* per local expert; one count per (rank, expert) pair (zbal_deepep.cpp:525-534) */
+        ZB_CHECK(op, "expertTokenNumsOut", expertTokenNumsOut, ZBAL_DATA_TYPE_INT64, ZBAL_DATA_TYPE_INT64, E / R);
+        ZB_CHECK(op, "epRecvCountsOut", epRecvCountsOut, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E * R);
+        ZB_CHECK(op, "putOffset", putOffset, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, E * R);
         /* an empty batch has empty per-token tensors (torch hands out a null pointer for them): only the counts are written */
         if (T > 0) {
             ZB_CHECK(op, "x", x, ZBAL_DATA_TYPE_BFP16, ZBAL_DATA_TYPE_FP16, T * H);
@@ -477,6 +480,29 @@ public:
                 ZB_CHECK(op, "dynamicScalesOut", dynamicScalesOut, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32,
                          quantMode == 1 ? T * K : T * K * (H / 128));
             }
+        }
+        if (R > 1) {
+            /*
+             * Every rank's expert ids and receive tensors sit at the same offset in that rank's window: the counts are
+             * taken from all ranks' ids, the rows go to the window of the rank that owns the expert. The receive
+             * tensors may be sized for what the rank receives; rows past them are dropped, not written.
+             */
+            const int64_t scalesPerRow = quantMode == 0 ? 0 : (quantMode == 1 ? 1 : H / 128);
+            int64_t destRows = T > 0 ? Numel(expandXOut) / H : 0;
+            if (T > 0 && scalesPerRow > 0 && Numel(dynamicScalesOut) / scalesPerRow < destRows)
+                destRows = Numel(dynamicScalesOut) / scalesPerRow;
+            const void *ids[ZBALHIP_MAX_REDUCE_PEERS] = {}, *dest[ZBALHIP_MAX_REDUCE_PEERS] = {}, *scale[ZBALHIP_MAX_REDUCE_PEERS] = {};
+            if (T > 0) {
+                if (!PeerCopies(op, expertIds->data, (size_t)(T * K) * 4, ids)) return Z_INVALID_PARAM;
+                if (!PeerCopies(op, expandXOut->data, (size_t)destRows * rowBytes, dest)) return Z_INVALID_PARAM;
+                if (scalesPerRow > 0 && !PeerCopies(op, dynamicScalesOut->data, (size_t)destRows * scalesPerRow * 4, scale))
+                    return Z_INVALID_PARAM;
+            }
+            return Launched(op, zbalhip_dispatch_low_latency_ranks(
+                                    x->data, x->dataType, (const int32_t *const *)ids, T, H, K, E, (int32_t)quantMode,
+                                    (int32_t)expertTokenNumsType, (void *const *)dest, (float *const *)scale, (int32_t)R,
+                                    (int32_t)me, destRows, (int32_t *)expandIdxOut->data, (int64_t *)expertTokenNumsOut->data,
+                                    (int32_t *)epRecvCountsOut->data, (int32_t *)putOffset->data, stream));
         }
         int64_t blocks = Numel(putOffset) / E;
         if (blocks > ZBALHIP_LAYOUT_MAX_BLOCKS) blocks = ZBALHIP_LAYOUT_MAX_BLOCKS;
@@ -495,7 +521,9 @@ public:
                               int64_t moeExpertNum, aclrtStream stream, int64_t) override
     {
         const char *op = "CombineLowlatency";
-        if (!SingleRank(op)) return Z_INVALID_PARAM;
+        const int64_t R = info_.groupSize, me = info_.myGroupRank;
+        ZBAL_VALIDATE_RETURN(R <= ZBALHIP_MAX_REDUCE_PEERS && moeExpertNum % R == 0,
+                             op << " failed as " << moeExpertNum << " experts do not split over a group of " << R, Z_INVALID_PARAM);
         int64_t T = 0, H = 0;
         if (!TokensShape(op, xOut, &T, &H)) return Z_INVALID_PARAM;
         ZBAL_VALIDATE_RETURN(expertIds->dim == 2 && expertIds->shape[0] == T, op << " failed as expertIds must be [tokens, topk]",
@@ -511,10 +539,13 @@ public:
         ZB_CHECK(op, "xOut", xOut, expandX->dataType, expandX->dataType, T * H);
         ZB_CHECK(op, "expertIds", expertIds, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
         ZB_CHECK(op, "expertIdx", expertIdx, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, T * K);
-        ZB_CHECK(op, "epSendCounts", epSendCounts, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, moeExpertNum);
+        ZB_CHECK(op, "epSendCounts", epSendCounts, ZBAL_DATA_TYPE_INT32, ZBAL_DATA_TYPE_INT32, moeExpertNum * R);
         ZB_CHECK(op, "expertScales", expertScales, ZBAL_DATA_TYPE_FP32, ZBAL_DATA_TYPE_FP32, T * K);
-        const void *src[1] = {expandX->data};
-        return Launched(op, zbalhip_combine(src, 1, 0, Numel(expandX) / H, expandX->dataType,
+        /* the expert outputs are read from the window of the rank that owns the expert (combine_low_latency.h:494-531) */
+        const int64_t srcRows = Numel(expandX) / H;
+        const void *src[ZBALHIP_MAX_REDUCE_PEERS];
+        if (!PeerCopies(op, expandX->data, (size_t)srcRows * H * 2, src)) return Z_INVALID_PARAM;
+        return Launched(op, zbalhip_combine(src, (int32_t)R, (int32_t)me, srcRows, expandX->dataType,
                                             (const int32_t *)epSendCounts->data, 1, (const float *)expertScales->data,
                                             (const int32_t *)expertIds->data, (const int32_t *)expertIdx->data, T, H, K,
                                             moeExpertNum, xOut->data, stream));

@@ -61,7 +61,8 @@ combine_kernel(PeerSource src, const int32_t *__restrict__ base, int base_inclus
                 if (rk < 0) masked = true;
                 else {
                     const int slot = e * src.ranks + src.my_rank;
-                    const int32_t b = base_inclusive ? (slot == 0 ? 0 : base[slot - 1]) : base[slot];
+                    /* running sums start anew with every rank's block of `experts` entries (low-latency counts) */
+                    const int32_t b = base_inclusive ? (slot % experts == 0 ? 0 : base[slot - 1]) : base[slot];
                     const int64_t row = (int64_t)b + rk;
                     if (row < src.rows_cap) {            /* never read past the window */
                         keep = true;
@@ -132,7 +133,6 @@ extern "C" int32_t zbalhip_combine(const void *const *y, int32_t ranks, int32_t 
         return ZBALHIP_INVALID;
     if (ranks <= 0 || ranks > ZBALHIP_MAX_REDUCE_PEERS || my_rank < 0 || my_rank >= ranks || experts % ranks != 0 || y_rows < 0)
         return ZBALHIP_INVALID;
-    if (base_is_inclusive && ranks != 1) return ZBALHIP_INVALID;
     PeerSource src = {};
     for (int r = 0; r < ranks; ++r) {
         if (!y[r]) return ZBALHIP_INVALID;

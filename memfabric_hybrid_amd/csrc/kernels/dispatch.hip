@@ -16,6 +16,10 @@ int32_t zbalhip_layout_ranges_internal(const int32_t *idx, int64_t tokens, int64
                                        const uint8_t *active_mask, int32_t *send_token_idx, int32_t *hist, int nblk,
                                        int tokens_per_block, hipStream_t st);
 
+int32_t zbalhip_ll_counts_internal(const int32_t *const *ids, int ranks, int me, int64_t tokens, int64_t topk,
+                                   int64_t experts, int32_t token_nums_type, int32_t *all_counts, int32_t *ep_recv_counts,
+                                   int64_t *expert_token_nums, hipStream_t st);
+
 int32_t zbalhip_layout_fused_internal(const int32_t *idx, int64_t tokens, int64_t experts, int64_t topk,
                                       int32_t token_nums_type, const uint8_t *active_mask, int32_t *send_token_idx,
                                       int32_t *incl_i32, int32_t *row_off, int64_t *counts_i64, int64_t *nums_typed,
@@ -46,8 +50,9 @@ struct PeerRows {
 __device__ __forceinline__ int64_t pick_row(const int32_t *__restrict__ base, int base_inclusive, const PeerRows &pr, int e,
                                             int32_t rank_in_expert)
 {
+    /* running sums start anew with every destination rank's block of `experts` entries (low-latency counts) */
     const int slot = e * pr.ranks + pr.my_rank;
-    const int32_t b = base_inclusive ? (slot == 0 ? 0 : base[slot - 1]) : base[slot];
+    const int32_t b = base_inclusive ? (slot % (pr.e_loc * pr.ranks) == 0 ? 0 : base[slot - 1]) : base[slot];
     const int64_t row = (int64_t)b + rank_in_expert;
     return row < pr.rows_cap ? row : -1;
 }
@@ -645,6 +650,43 @@ extern "C" int32_t zbalhip_dispatch_low_latency(const void *x, int32_t x_dtype, 
     if (rc != ZBALHIP_OK) return rc;
     return permute_launch(x, x_dtype, expert_ids, expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk, experts, q,
                           single_window(expand_x, dynamic_scales, experts, tokens * topk), st);
+}
+
+extern "C" int32_t zbalhip_dispatch_low_latency_ranks(const void *x, int32_t x_dtype, const int32_t *const *expert_ids,
+                                                      int64_t tokens, int64_t hidden, int64_t topk, int64_t experts,
+                                                      int32_t quant_mode, int32_t token_nums_type, void *const *expand_x,
+                                                      float *const *dynamic_scales, int32_t ranks, int32_t my_rank,
+                                                      int64_t dest_rows, int32_t *expand_idx, int64_t *expert_token_nums,
+                                                      int32_t *ep_recv_counts, int32_t *all_counts, void *stream)
+{
+    if (!expert_ids || !expert_token_nums || !ep_recv_counts || !all_counts) return ZBALHIP_INVALID;
+    if (experts <= 0 || experts > 1024 || topk <= 0 || tokens < 0 || tokens * topk > 0x7fffffff || quant_mode < 0 ||
+        quant_mode > 2 || dest_rows < 0)
+        return ZBALHIP_INVALID;
+    if (ranks <= 0 || ranks > ZBALHIP_MAX_REDUCE_PEERS || my_rank < 0 || my_rank >= ranks || experts % ranks != 0)
+        return ZBALHIP_INVALID;
+    if (tokens > 0 && (!x || !expand_x || !expand_idx || (quant_mode != 0 && !dynamic_scales))) return ZBALHIP_INVALID;
+    PeerRows pr = {};
+    for (int r = 0; r < ranks; ++r) {
+        if (tokens > 0 && (!expert_ids[r] || !expand_x[r] || (quant_mode != 0 && !dynamic_scales[r]))) return ZBALHIP_INVALID;
+        pr.dest[r] = tokens > 0 ? (uint8_t *)expand_x[r] : nullptr;
+        pr.scale[r] = (tokens > 0 && quant_mode != 0) ? dynamic_scales[r] : nullptr;
+    }
+    pr.ranks = ranks;
+    pr.my_rank = my_rank;
+    pr.e_loc = (int)(experts / ranks);
+    pr.rows_cap = dest_rows;
+    hipStream_t st = (hipStream_t)stream;
+    int32_t rc = zbalhip_ll_counts_internal(expert_ids, ranks, my_rank, tokens, topk, experts, token_nums_type, all_counts,
+                                            ep_recv_counts, expert_token_nums, st);
+    if (rc != ZBALHIP_OK || tokens == 0) return rc;
+    /* the rank of each of my picks among my own earlier picks of the same expert */
+    rc = zbalhip_layout_fused_internal(expert_ids[my_rank], tokens, experts, topk, 1, nullptr, expand_idx, nullptr, nullptr,
+                                       nullptr, nullptr, st);
+    if (rc != ZBALHIP_OK) return rc;
+    const int q = quant_mode == 0 ? QM_COPY : (quant_mode == 1 ? QM_INT8_NOEPS : QM_FP8);
+    return permute_launch(x, x_dtype, expert_ids[my_rank], expand_idx, ep_recv_counts, 1, nullptr, tokens, hidden, topk,
+                          experts, q, pr, st);
 }
 
 extern "C" int32_t zbalhip_fused_permute_quant(const void *x, int32_t x_dtype, const int32_t *expert_ids,

@@ -398,6 +398,66 @@ notify_ranks_kernel(CountsOfRanks counts, int ranks, int me, int experts, int to
     }
 }
 
+/*
+ * Counts of the low-latency dispatch for a group of R ranks, from the point of view of rank `me` (reference
+ * zbal_kernel_dispatch_low_latency.h: every rank's per-expert counts gathered into allExpertTokenNums :344-345,
+ * ReorderRecvDataOutput :690-713, WaitNotify :641-688). ids.p[s] is rank s's [tokens, topk] expert ids, read where
+ * they lie in that rank's window (the reference's ranks push their counts to each other and wait for flags; on one
+ * GPU the inputs of all modelled ranks are in place before any of them is launched). all_counts[s * E + e] = picks
+ * of expert e by rank s; ep_recv_counts[r * E + le * R + s] = INCLUSIVE running sum, per destination rank r, over
+ * its local experts le and, within an expert, the source ranks s (a consumer takes index i's start from entry i - 1,
+ * 0 at the start of a rank's block); expert_token_nums[le] = rows rank `me` receives for its local expert le
+ * (type 1) or their running sum (type 0). One block, one thread per (local expert, source rank) pair.
+ */
+struct IdsOfRanks {
+    const int32_t *p[ZBALHIP_MAX_REDUCE_PEERS];
+};
+
+__global__ void __launch_bounds__(ZB_MAX_EXPERTS)
+ll_counts_kernel(IdsOfRanks ids, int ranks, int me, int tokens, int topk, int experts, int token_nums_type,
+                 int32_t *__restrict__ all_counts, int32_t *__restrict__ ep_recv_counts,
+                 int64_t *__restrict__ expert_token_nums)
+{
+    __shared__ int32_t hist[ZB_MAX_EXPERTS];
+    __shared__ int32_t mine[ZB_MAX_EXPERTS];
+    __shared__ int32_t wsum[ZB_MAX_EXPERTS / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, nwaves = blockDim.x >> 6;
+    const int n = tokens * topk, e_loc = experts / ranks;
+    for (int s = 0; s < ranks; ++s) {
+        for (int e = tid; e < experts; e += blockDim.x) hist[e] = 0;
+        __syncthreads();
+        for (int i = tid; i < n; i += blockDim.x) {
+            const int e = ids.p[s][i];
+            if (e >= 0 && e < experts) atomicAdd(&hist[e], 1);
+        }
+        __syncthreads();
+        for (int e = tid; e < experts; e += blockDim.x) all_counts[s * experts + e] = hist[e];
+        __syncthreads();
+    }
+    for (int r = 0; r < ranks; ++r) {
+        const int le = tid / ranks, s = tid - le * ranks;
+        const int32_t c = tid < experts ? all_counts[s * experts + r * e_loc + le] : 0;
+        int32_t incl = c;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int32_t o = __shfl_up(incl, off, 64);
+            if (lane >= off) incl += o;
+        }
+        if (lane == 63) wsum[wave] = incl;
+        __syncthreads();
+        for (int w = 0; w < wave && w < nwaves; ++w) incl += wsum[w];
+        if (tid < experts) {
+            ep_recv_counts[r * experts + tid] = incl;
+            if (r == me) mine[tid] = incl;
+        }
+        __syncthreads();
+    }
+    for (int le = tid; le < e_loc; le += blockDim.x) {
+        const int32_t hi = mine[(le + 1) * ranks - 1], lo = le ? mine[le * ranks - 1] : 0;
+        expert_token_nums[le] = token_nums_type == 0 ? (int64_t)hi : (int64_t)(hi - lo);
+    }
+}
+
 /* ---- router ----------------------------------------------------------------- */
 
 /*
@@ -562,6 +622,18 @@ int32_t zbalhip_layout_ranges_internal(const int32_t *idx, int64_t tokens, int64
     layout_ranges_kernel<int32_t><<<nblk, ZB_FUSED_THREADS, 0, st>>>(idx, (int)tokens, (int)topk, (int)experts,
                                                                     tokens_per_block, ceil_log2(experts), active_mask,
                                                                     send_token_idx, hist);
+    return zbalhip_check_launch();
+}
+
+int32_t zbalhip_ll_counts_internal(const int32_t *const *ids, int ranks, int me, int64_t tokens, int64_t topk,
+                                   int64_t experts, int32_t token_nums_type, int32_t *all_counts, int32_t *ep_recv_counts,
+                                   int64_t *expert_token_nums, hipStream_t st)
+{
+    IdsOfRanks all = {};
+    for (int r = 0; r < ranks; ++r) all.p[r] = ids[r];
+    const int threads = (int)((experts + 63) / 64 * 64);
+    ll_counts_kernel<<<1, threads, 0, st>>>(all, ranks, me, (int)tokens, (int)topk, (int)experts, token_nums_type, all_counts,
+                                            ep_recv_counts, expert_token_nums);
     return zbalhip_check_launch();
 }
 

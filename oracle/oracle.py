@@ -195,6 +195,41 @@ def combine_low_latency(expand_x, dtype, expert_ids, expand_idx, ep_send_counts,
     return out
 
 
+def ll_counts(ids_all, E, me, token_nums_type=1):
+    """ids_all [R, T, K] -> (all_counts [R, E], ep_recv_counts [R * E], expert_token_nums [E / R]) as rank `me` sees them."""
+    ids = np.ascontiguousarray(ids_all, dtype=np.int32)
+    R, T, K = ids.shape
+    allc = np.zeros((R, E), dtype=np.int32)
+    recv = np.zeros(R * E, dtype=np.int32)
+    nums = np.zeros(E // R, dtype=np.int64)
+    lib().zo_ll_counts(_p(ids), _i64(R), _i64(me), _i64(T), _i64(K), _i64(E), _i32(token_nums_type), _p(allc), _p(recv), _p(nums))
+    return allc, recv, nums
+
+
+def dispatch_low_latency_ranks(x, x_dtype, expert_ids, E, R, me, quant_mode, ep_recv_counts, windows_x, windows_scale):
+    """Rank `me` writes its rows into windows_x [R, rows_cap, H] / windows_scale [R, rows_cap(, H/128)] in place; returns expand_idx."""
+    T, H = x.shape
+    K = expert_ids.shape[1]
+    eidx = np.zeros((T, K), dtype=np.int32)
+    lib().zo_dispatch_low_latency_ranks(_p(x), _i32(x_dtype), _p(np.ascontiguousarray(expert_ids, dtype=np.int32)), _i64(T),
+                                        _i64(H), _i64(K), _i64(E), _i64(R), _i64(me), _i32(quant_mode),
+                                        _p(np.ascontiguousarray(ep_recv_counts, dtype=np.int32)), _i64(windows_x.shape[1]),
+                                        _p(windows_x), _p(windows_scale), _p(eidx))
+    return eidx
+
+
+def combine_low_latency_ranks(windows_y, dtype, expert_ids, expand_idx, ep_send_counts, w, E, R, me):
+    T, K = expert_ids.shape
+    H = windows_y.shape[2]
+    out = np.zeros((T, H), dtype=np.uint16)
+    lib().zo_combine_low_latency_ranks(_p(windows_y), _i32(dtype), _p(np.ascontiguousarray(expert_ids, dtype=np.int32)),
+                                       _p(np.ascontiguousarray(expand_idx, dtype=np.int32)),
+                                       _p(np.ascontiguousarray(ep_send_counts, dtype=np.int32)),
+                                       _p(np.ascontiguousarray(w, dtype=np.float32)), _i64(T), _i64(H), _i64(K), _i64(E),
+                                       _i64(R), _i64(me), _i64(windows_y.shape[1]), _p(out))
+    return out
+
+
 def fused_permute_quant(x, x_dtype, expert_ids, smooth, E, mode):
     T, H = x.shape
     K = expert_ids.shape[1]

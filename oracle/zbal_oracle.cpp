@@ -509,6 +509,124 @@ ZO_API void zo_combine_low_latency(const uint16_t *expand_x, int32_t dtype, cons
     zo_combine(expand_x, dtype, base.data(), w, expert_ids, expand_idx, T, H, K, E, 1, 0, out);
 }
 
+/*
+ * The low-latency pair for a group of R ranks, from the point of view of rank `me`
+ * (OPS/dispatch_combine_low_latency/zbal_kernel_dispatch_low_latency.h: counts of all ranks gathered into
+ * allExpertTokenNums :344-345; ReorderRecvDataOutput :690-713 builds, per destination rank r, the INCLUSIVE running sum
+ * over (local expert le, source rank s) at [r * E + le * R + s]; WaitNotify :641-688 derives the receiving rank's
+ * expertTokenNums from its own block; SendToMoeExpert :760-844 puts pick (t, k) of expert e into the window of rank
+ * e / E_loc at row start(e * R + me) + expand_idx, start(i) = i % E == 0 ? 0 : counts[i - 1]).
+ * ids_all [R][T][K]: every rank's expert ids (all ranks with the same T and K).
+ */
+ZO_API void zo_ll_counts(const int32_t *ids_all, int64_t R, int64_t me, int64_t T, int64_t K, int64_t E,
+                         int32_t token_nums_type, int32_t *all_counts, int32_t *ep_recv_counts,
+                         int64_t *expert_token_nums)
+{
+    const int64_t e_loc = E / R;
+    std::fill(all_counts, all_counts + R * E, 0);
+    for (int64_t s = 0; s < R; ++s)
+        for (int64_t i = 0; i < T * K; ++i) {
+            const int64_t e = ids_all[s * T * K + i];
+            if (e >= 0 && e < E) all_counts[s * E + e] += 1;
+        }
+    for (int64_t r = 0; r < R; ++r) {
+        int32_t prefix = 0;
+        for (int64_t le = 0; le < e_loc; ++le)
+            for (int64_t s = 0; s < R; ++s) {
+                prefix += all_counts[s * E + r * e_loc + le];
+                ep_recv_counts[r * E + le * R + s] = prefix;
+            }
+    }
+    int64_t sums = 0;
+    for (int64_t le = 0; le < e_loc; ++le) {
+        const int64_t cur = R * (le + 1) - 1;
+        const int64_t before = le == 0 ? 0 : ep_recv_counts[me * E + cur - R];
+        const int64_t here = ep_recv_counts[me * E + cur] - before;
+        sums = (token_nums_type == 0 ? sums : 0) + here;
+        expert_token_nums[le] = sums;
+    }
+}
+
+/*
+ * Rank `me` sends its tokens: windows_x / windows_scale are the R receive windows one after the other (rows_cap rows
+ * each); only the rows this rank writes are touched. expand_idx = rank of each pick among this rank's earlier picks
+ * of the same expert (-1 for an invalid id).
+ */
+ZO_API void zo_dispatch_low_latency_ranks(const uint16_t *x, int32_t x_dtype, const int32_t *expert_ids, int64_t T,
+                                          int64_t H, int64_t K, int64_t E, int64_t R, int64_t me, int32_t quant_mode,
+                                          const int32_t *ep_recv_counts, int64_t rows_cap, void *windows_x,
+                                          float *windows_scale, int32_t *expand_idx)
+{
+    const int64_t e_loc = E / R;
+    std::vector<int32_t> cnt(E, 0);
+    for (int64_t i = 0; i < T * K; ++i) {
+        const int64_t e = expert_ids[i];
+        if (e < 0 || e >= E) { expand_idx[i] = -1; continue; }
+        expand_idx[i] = cnt[e]++;
+    }
+    std::vector<int8_t> q(H);
+    std::vector<uint8_t> q8(H);
+    std::vector<float> v(H), sc(H / 128 + 1);
+    for (int64_t t = 0; t < T; ++t) {
+        bool done = false;
+        float scale = 0.0f;
+        for (int64_t k = 0; k < K; ++k) {
+            const int64_t e = expert_ids[t * K + k];
+            if (e < 0 || e >= E) continue;
+            const int64_t idx = e * R + me;
+            const int64_t start = idx % E == 0 ? 0 : ep_recv_counts[idx - 1];
+            const int64_t row = start + expand_idx[t * K + k];
+            if (row >= rows_cap) continue;
+            const int64_t wrow = (e / e_loc) * rows_cap + row;
+            if (quant_mode == 0) {
+                std::memcpy(static_cast<uint16_t *>(windows_x) + wrow * H, x + t * H, size_t(H) * 2);
+            } else if (quant_mode == 1) {
+                if (!done) { quant_row_int8(x + t * H, x_dtype, H, nullptr, 1, q.data(), &scale); done = true; }
+                std::memcpy(static_cast<int8_t *>(windows_x) + wrow * H, q.data(), size_t(H));
+                windows_scale[wrow] = scale;
+            } else {
+                if (!done) {
+                    for (int64_t j = 0; j < H; ++j) v[j] = half_like_to_f32(x[t * H + j], x_dtype);
+                    quant_row_fp8(v.data(), H, q8.data(), sc.data());
+                    done = true;
+                }
+                std::memcpy(static_cast<uint8_t *>(windows_x) + wrow * H, q8.data(), size_t(H));
+                std::memcpy(windows_scale + wrow * (H / 128), sc.data(), size_t(H / 128) * 4);
+            }
+        }
+    }
+}
+
+/*
+ * Rank `me` combines: zbal_kernel_combine_low_latency.h:494-531 (row of pick (t, k) of expert e: window e / E_loc, row
+ * start(e * R + me) + expand_idx; Muls then Add in fp32, one rounding). windows_y: the R windows one after the other.
+ */
+ZO_API void zo_combine_low_latency_ranks(const uint16_t *windows_y, int32_t dtype, const int32_t *expert_ids,
+                                         const int32_t *expand_idx, const int32_t *ep_send_counts, const float *w,
+                                         int64_t T, int64_t H, int64_t K, int64_t E, int64_t R, int64_t me,
+                                         int64_t rows_cap, uint16_t *out)
+{
+    const int64_t e_loc = E / R;
+#pragma omp parallel for schedule(static)
+    for (int64_t t = 0; t < T; ++t) {
+        std::vector<float> acc(H, 0.0f);
+        for (int64_t k = 0; k < K; ++k) {
+            const int64_t e = expert_ids[t * K + k];
+            if (e < 0 || e >= E) continue;
+            const int64_t idx = e * R + me;
+            const int64_t row = (idx % E == 0 ? 0 : ep_send_counts[idx - 1]) + expand_idx[t * K + k];
+            if (row >= rows_cap) continue;
+            const uint16_t *src = windows_y + ((e / e_loc) * rows_cap + row) * H;
+            const float wk = w[t * K + k];
+            for (int64_t j = 0; j < H; ++j) {
+                const float tmp = half_like_to_f32(src[j], dtype) * wk;
+                acc[j] = acc[j] + tmp;
+            }
+        }
+        for (int64_t j = 0; j < H; ++j) out[t * H + j] = f32_to_half_like(acc[j], dtype);
+    }
+}
+
 /* ---- grouped GEMMs ------------------------------------------------------ */
 
 /*

@@ -78,6 +78,12 @@ class OuterAbi:
     def combine(self, r, *a):
         return self.lib.zbal_combine_normal(*a, self.comms[r], capi.stream_ptr(), 0)
 
+    def ll_dispatch(self, r, *a):
+        return self.lib.zbal_dispatch_low_latency(*a, self.comms[r], capi.stream_ptr(), 0)
+
+    def ll_combine(self, r, *a):
+        return self.lib.zbal_combine_low_latency(*a, self.comms[r], capi.stream_ptr(), 0)
+
 
 class KernelSeam:
     """ZBALOp* launchers with a CommGroupInfo per modelled rank: the peers are localDeviceMemSize bytes apart."""
@@ -106,6 +112,12 @@ class KernelSeam:
 
     def combine(self, r, *a):
         return self.fn["ZBALOpCombineNormal"](*a, False, capi.stream_ptr(), ctypes.byref(self.infos[r]), 0)
+
+    def ll_dispatch(self, r, *a):
+        return self.fn["ZBALOpDispatchLowLatency"](*a, capi.stream_ptr(), ctypes.byref(self.infos[r]), 0)
+
+    def ll_combine(self, r, *a):
+        return self.fn["ZBALOpCombineLowLatency"](*a, capi.stream_ptr(), ctypes.byref(self.infos[r]), 0)
 
 
 @pytest.mark.parametrize("api_cls", [OuterAbi, KernelSeam])
@@ -393,3 +405,76 @@ def test_fused_and_all_reduce_through_the_launcher_seam(buf):
         assert rc == 0, capi.last_error()
         assert torch.equal(out, ref_sum)
         assert gi.waitSymbol == 1
+
+
+@pytest.mark.parametrize("api_cls", [OuterAbi, KernelSeam])
+@pytest.mark.parametrize("R,quant,T,K,E,H,nums_type", [(1, 1, 48, 4, 16, 256, 1), (2, 0, 48, 4, 16, 256, 0), (4, 1, 33, 8, 32, 512, 1),
+                                                        (4, 2, 40, 3, 8, 1024, 0), (2, 1, 700, 8, 64, 256, 1)])
+def test_low_latency_pair_over_modelled_ranks(buf, api_cls, R, quant, T, K, E, H, nums_type):
+    """Low-latency dispatch and combine over R modelled ranks: counts from every rank's ids, rows into the window of
+    the rank that owns the expert at the running-sum offsets ep_recv_counts[r * E + le * R + src], combine reading them
+    back from there. Bit for bit against the oracle's R-rank functions, through both ABIs."""
+    lib = buf.lib
+    ti, ref = capi.tensor_info, ctypes.byref
+    rows_cap = R * T * K
+    qbytes = 2 if quant == 0 else 1
+    spr = {0: 1, 1: 1, 2: H // 128}[quant]
+    layout = [("ids", T * K * 4, torch.int32), ("recv_x", rows_cap * H * qbytes, torch.uint8),
+              ("recv_scale", rows_cap * spr * 4, torch.float32), ("expert_out", rows_cap * H * 2, torch.bfloat16)]
+    wins = Window.make(layout, R)
+    api = api_cls(lib, wins, "ll%d_%d_%d_%d" % (R, quant, T, H))
+    try:
+        ids_all = rng(300 + R).integers(-1, E + 1, size=(R, T, K)).astype(np.int32)
+        xs = [bf16_normal((T, H), 310 + r) for r in range(R)]
+        w = [rng(320 + r).uniform(0, 1, (T, K)).astype(np.float32) for r in range(R)]
+        for r in range(R):
+            wins[r]["ids"].copy_(torch.from_numpy(ids_all[r].reshape(-1)))
+        recv_dt = {0: capi.DT_BF16, 1: capi.DT_INT8, 2: capi.DT_FP8_E4M3}[quant]
+        out = []
+        for r in range(R):
+            x_d = torch.from_numpy(xs[r]).view(torch.int16).view(torch.bfloat16).cuda()
+            eidx = torch.full((T, K), -9, dtype=torch.int32, device="cuda")
+            nums = torch.full((E // R,), -9, dtype=torch.int64, device="cuda")
+            recv = torch.full((R * E,), -9, dtype=torch.int32, device="cuda")
+            put = torch.full((max(R, 2) * E,), -9, dtype=torch.int32, device="cuda")
+            status = torch.zeros(R * E, dtype=torch.float32, device="cuda")
+            rc = api.ll_dispatch(r, ref(ti(x_d)), ref(ti(wins[r]["ids"], shape=(T, K))), E, 0, 0, quant, 0, 0, nums_type,
+                                 ref(ti(wins[r]["recv_x"], dtype=recv_dt, shape=(rows_cap, H))), ref(ti(wins[r]["recv_scale"])),
+                                 ref(ti(eidx)), ref(ti(nums)), ref(ti(recv)), ref(ti(put)), ref(ti(status)))
+            assert rc == 0, capi.last_error()
+            out.append((eidx, nums, recv, put))
+        torch.cuda.synchronize()
+        np_x = np.zeros((R, rows_cap, H), dtype=np.uint16 if quant == 0 else np.uint8)
+        np_s = np.zeros((R, rows_cap, spr) if quant == 2 else (R, rows_cap), dtype=np.float32)
+        for r in range(R):
+            allc, o_recv, o_nums = zo.ll_counts(ids_all, E, r, nums_type)
+            o_eidx = zo.dispatch_low_latency_ranks(xs[r], zo.DT_BF16, ids_all[r], E, R, r, quant, o_recv, np_x, np_s)
+            eidx, nums, recv, put = out[r]
+            assert np.array_equal(host(eidx), o_eidx) and np.array_equal(host(nums), o_nums)
+            assert np.array_equal(host(recv), o_recv)
+            if R > 1:
+                assert np.array_equal(host(put)[:R * E], allc.reshape(-1))
+        e_loc = E // R
+        for d in range(R):
+            n_rows = int(zo.ll_counts(ids_all, E, d, 1)[2].sum())
+            got = host(wins[d]["recv_x"]).reshape(rows_cap, H * qbytes)
+            got = got.view(np.uint16) if quant == 0 else got
+            assert np.array_equal(got[:n_rows], np_x[d, :n_rows]), "rows in window %d" % d
+            if quant != 0:
+                assert np.array_equal(host(wins[d]["recv_scale"]).reshape(rows_cap, spr)[:n_rows], np_s[d].reshape(rows_cap, spr)[:n_rows])
+        # ---- combine: the expert outputs sit in the windows the rows were dispatched to
+        y = np.stack([bf16_normal((rows_cap, H), 330 + d) for d in range(R)])
+        for d in range(R):
+            wins[d]["expert_out"].copy_(torch.from_numpy(y[d].reshape(-1)).view(torch.int16).view(torch.bfloat16))
+        for r in range(R):
+            eidx, nums, recv, put = out[r]
+            res = torch.zeros((T, H), dtype=torch.bfloat16, device="cuda")
+            ids32 = torch.from_numpy(ids_all[r]).cuda()
+            rc = api.ll_combine(r, ref(ti(wins[r]["expert_out"], shape=(rows_cap, H))), ref(ti(ids32)), ref(ti(eidx)), ref(ti(recv)),
+                                ref(ti(torch.from_numpy(w[r]).cuda())), ref(ti(res)), E)
+            assert rc == 0, capi.last_error()
+            want = zo.combine_low_latency_ranks(y, zo.DT_BF16, ids_all[r], host(eidx), host(recv), w[r], E, R, r)
+            assert np.array_equal(host(res), want), "combine of rank %d" % r
+    finally:
+        torch.cuda.synchronize()
+        api.close()

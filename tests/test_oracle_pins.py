@@ -141,6 +141,73 @@ def test_notify_multi_rank_closed_form():
         assert np.array_equal(per_exp, counts[:, me * eloc:(me + 1) * eloc].sum(0))
 
 
+def test_low_latency_counts_over_ranks_closed_form():
+    """zo_ll_counts against numpy: all_counts is a bincount per rank; every destination rank's block of ep_recv_counts
+    is the inclusive cumsum of its local experts' counts taken expert by expert and, within one, source rank by
+    source rank (starting at 0 for every rank); expert_token_nums are the column sums of the receiving rank's experts
+    (type 1) or their running sum (type 0). At R = 1 the block is zo_dispatch_low_latency's ep_recv_counts."""
+    R, T, K, E = 4, 37, 3, 16
+    ids = rng(70).integers(-1, E + 1, size=(R, T, K)).astype(np.int32)
+    e_loc = E // R
+    want_all = np.stack([np.bincount(ids[s][(ids[s] >= 0) & (ids[s] < E)], minlength=E) for s in range(R)])
+    for me in range(R):
+        for typ in (0, 1):
+            allc, recv, nums = zo.ll_counts(ids, E, me, typ)
+            assert np.array_equal(allc, want_all)
+            for r in range(R):
+                seq = want_all[:, r * e_loc:(r + 1) * e_loc].T.reshape(-1)          # le-major, src-minor
+                assert np.array_equal(recv[r * E:(r + 1) * E], np.cumsum(seq))
+            per = want_all[:, me * e_loc:(me + 1) * e_loc].sum(0)
+            assert np.array_equal(nums, np.cumsum(per) if typ == 0 else per)
+    one = ids[:1]
+    x = zo.f32_to_bf16(rng(71).standard_normal((T, 128)).astype(np.float32))
+    _, _, eidx1, nums1, counts1 = zo.dispatch_low_latency(x, zo.DT_BF16, one[0], E, 0, T * K)
+    allc, recv, nums = zo.ll_counts(one, E, 0, 1)
+    assert np.array_equal(recv, counts1) and np.array_equal(nums, nums1)
+
+
+def test_low_latency_dispatch_and_combine_over_ranks():
+    """R ranks dispatch into R windows and combine back: every window ends up densely packed in (local expert,
+    source rank, pick order) order with the rows of the tokens that picked the expert -- checked row by row against a
+    direct construction --, no row is written twice, and combine(dispatch(x)) = x * sum of the valid picks' weights
+    (the reference test's round trip, test_low_latency.py:146-155). At R = 1 both functions equal the one-rank ones."""
+    R, T, H, K, E = 3, 29, 128, 4, 12
+    e_loc = E // R
+    ids = np.stack([np.stack([rng(80 + s * 100 + t).permutation(E + 2)[:K] - 1 for t in range(T)]) for s in range(R)]).astype(np.int32)
+    xs = [zo.f32_to_bf16(rng(90 + s).standard_normal((T, H)).astype(np.float32)) for s in range(R)]
+    ws = [rng(95 + s).uniform(0, 1, (T, K)).astype(np.float32) for s in range(R)]
+    rows_cap = R * T * K
+    win = np.zeros((R, rows_cap, H), dtype=np.uint16)
+    scale = np.zeros((R, rows_cap), dtype=np.float32)
+    _, recv, _ = zo.ll_counts(ids, E, 0)
+    eidx = [zo.dispatch_low_latency_ranks(xs[s], zo.DT_BF16, ids[s], E, R, s, 0, recv, win, scale) for s in range(R)]
+    for d in range(R):                       # direct construction of window d
+        row = 0
+        for le in range(e_loc):
+            for s in range(R):
+                for t in range(T):
+                    for k in range(K):
+                        if ids[s, t, k] == d * e_loc + le:
+                            assert np.array_equal(win[d, row], xs[s][t]), (d, le, s, t, k)
+                            row += 1
+        assert not win[d, row:].any()
+    for s in range(R):
+        out = zo.combine_low_latency_ranks(win, zo.DT_BF16, ids[s], eidx[s], recv, ws[s], E, R, s)
+        valid = (ids[s] >= 0) & (ids[s] < E)
+        want = zo.bf16_to_f32(xs[s]) * (ws[s] * valid).sum(1, keepdims=True)
+        got = zo.bf16_to_f32(out)
+        for t in range(T):
+            assert calc_diff(got[t], want[t]) < 1e-5
+    # one rank: the general functions are the one-rank ones
+    ex1, _, eidx1, _, counts1 = zo.dispatch_low_latency(xs[0], zo.DT_BF16, ids[0], E, 0, T * K)
+    _, recv1, _ = zo.ll_counts(ids[:1], E, 0)
+    w1 = np.zeros((1, T * K, H), dtype=np.uint16)
+    e1 = zo.dispatch_low_latency_ranks(xs[0], zo.DT_BF16, ids[0], E, 1, 0, 0, recv1, w1, np.zeros((1, T * K), dtype=np.float32))
+    assert np.array_equal(w1[0], ex1) and np.array_equal(e1, eidx1) and np.array_equal(recv1, counts1)
+    assert np.array_equal(zo.combine_low_latency_ranks(w1, zo.DT_BF16, ids[0], e1, recv1, ws[0], E, 1, 0),
+                          zo.combine_low_latency(ex1, zo.DT_BF16, ids[0], eidx1, counts1, ws[0], E))
+
+
 # ---- quantising dispatch --------------------------------------------------------
 
 def make_dispatch(T, H, K, E, seed):
