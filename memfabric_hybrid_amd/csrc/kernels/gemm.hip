@@ -101,9 +101,9 @@ __device__ __forceinline__ uint32_t pack4_e4m3(float a, float b, float c, float 
  * those rows (zb_block_row_channel), so the sub-tiles nt = 2s and 2s+1 together are eight consecutive channels.
  * `lds_rowmax` is [2][tile_rows] floats of scratch for the row maxima of the two channel halves (GMM1 only).
  */
-template <int MODE, bool GMM1, int OUT_DT, int RG>
-__device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &tc, f32x4 (&accf)[4][8],
-                                         i32x4 (&acci)[4][8], int row_begin, int row_end, int wm, int wn, int lane,
+template <int MODE, bool GMM1, int OUT_DT, int RG, int MTM>
+__device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &tc, f32x4 (&accf)[MTM][8],
+                                         i32x4 (&acci)[MTM][8], int row_begin, int row_end, int wm, int wn, int lane,
                                          float *lds_rowmax, int tile_rows, const float *es)
 {
     /*
@@ -121,7 +121,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
     if constexpr (!GMM1) {
         uint16_t *y = (uint16_t *)p.out;
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < MTM; ++mt) {
             const int row = row_begin + (RG * mt + wm) * 16 + frag_row;
             if (row >= row_end) continue;
             float xs = 1.0f;
@@ -165,10 +165,10 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
         }
     } else {
         /* SwiGLU on gate sub-tile nt and up sub-tile nt+4: columns j = n_tile*128 + wn*64 + 32*(nt/2) + q8 + 4*(nt%2) + i */
-        float sg[4][4][4];
-        float rmax[4];
+        float sg[MTM][4][4];
+        float rmax[MTM];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < MTM; ++mt) {
             /*
              * A 16-row sub-tile past the tile's end holds nothing (the K loop left it out as well): its SwiGLU, which is
              * most of this epilogue's arithmetic (an exact exp and a division per value in the int modes), is skipped.
@@ -220,7 +220,7 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
         }
         __syncthreads();
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt) {
+        for (int mt = 0; mt < MTM; ++mt) {
             const int lr = (RG * mt + wm) * 16 + frag_row;
             const int row = row_begin + lr;
             const float amax_tile = fmaxf(lds_rowmax[lr], lds_rowmax[tile_rows + lr]);
@@ -283,21 +283,27 @@ constexpr int D_MAX_EXPERTS = 1024;
 /* WRB = bytes of one weight row per slab: 128 (8-bit) or 64 (packed int4) */
 template <int TM, int NSTAGE, int WRB>
 struct DmaShape {
-    static constexpr int ROW_GROUPS = TM / 64;
+    static constexpr int ROW_GROUPS = TM > 256 ? 4 : TM / 64;
+    static constexpr int MTM = (TM / 16 + ROW_GROUPS - 1) / ROW_GROUPS;   /* 16-row sub-tiles per wave, at most: 4, or 5 in the 288-row shape */
     static constexpr int NW = ROW_GROUPS * 2;
     static constexpr int THREADS = NW * 64;
     static constexpr int A_BYTES = TM * BKB;
     static constexpr int W_BYTES = BN * WRB;
     static constexpr int STAGE_BYTES = A_BYTES + W_BYTES;
     static constexpr int HALF_BLOCKS = 128 * WRB / 1024;   /* 1 KiB blocks per 128-channel half: 16 or 8 */
-    static constexpr int A_PARTS = A_BYTES / 1024 / NW;    /* 1 KiB blocks of the A tile per wave (4) */
+    static constexpr int A_PARTS = (A_BYTES / 1024 + NW - 1) / NW;   /* 1 KiB blocks of the A tile per wave: 4 (288 rows: 5, the last for half of the waves) */
     static constexpr int W_PARTS = W_BYTES / 1024 / NW;    /* 1 KiB blocks of the W tile per wave (2, 4 or 8) */
     static constexpr int PARTS = W_PARTS > A_PARTS ? W_PARTS : A_PARTS;
     static constexpr bool TWO_PHASE = TM == 256;            /* the tiles of short experts run after all the others (see the kernel) */
-    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + 4 * D_MAX_KB * 4 +
+    /* two buffers of per-tile scales, floats each: fp8 2 x D_MAX_KB weight block scales; W8A8 256 channel + TM token scales */
+    static constexpr int SW_STRIDE = TM > 256 ? 576 : 2 * D_MAX_KB;
+    static constexpr int SW_BYTES = 2 * SW_STRIDE * 4;
+    static_assert(SW_STRIDE >= 2 * D_MAX_KB && SW_STRIDE >= 256 + TM, "scale buffer too small");
+    static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + SW_BYTES +
                                      2 * (D_MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0) +
                                      (TWO_PHASE ? D_MAX_EXPERTS * 2 + (D_MAX_EXPERTS + 1) * 4 : 0);
-    static_assert(A_PARTS == 4 && PARTS % 4 == 0, "the issue schedule hands out a slab in four quarters");
+    static_assert((A_PARTS == 4 && PARTS % 4 == 0) || (TM == 288 && NSTAGE == 2 && PARTS == 5),
+                  "the issue schedule hands out a slab in four quarters (the 288-row shape: a fifth part with the last quarter)");
     static_assert(NW <= HALF_BLOCKS && HALF_BLOCKS % NW == 0, "a wave's W blocks must not straddle a weight half");
     static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
 };
@@ -384,7 +390,7 @@ template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE, bool WSTREAM>
  * the slabs in flight (1.7x slower than the 256-row shape on few-row experts). The int flavours fit 256 and are
  * a little faster compiled for it.
  */
-__global__ void __launch_bounds__(TM * 2, (TM == 128 && MODE == MODE_FP8) ? 1 : 2)
+__global__ void __launch_bounds__(TM > 256 ? 512 : TM * 2, (TM == 128 && MODE == MODE_FP8) ? 1 : 2)
 grouped_gemm_dma_kernel(GemmParams p)
 {
     static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8 || MODE == MODE_W4A8, "unknown mode");
@@ -398,8 +404,9 @@ grouped_gemm_dma_kernel(GemmParams p)
     extern __shared__ __attribute__((aligned(1024))) uint8_t smem[];
     float *lds_sa = reinterpret_cast<float *>(smem + NSTAGE * STAGE_BYTES);   /* [NSTAGE][TM] */
     float *lds_rowmax = lds_sa + NSTAGE * TM;                                 /* [2][TM] */
-    float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2 tiles][2][D_MAX_KB] fp8 weight block scales */
-    int *lds_mtp = reinterpret_cast<int *>(lds_sw + 4 * D_MAX_KB);            /* [experts + 1] tiles of TM rows before expert e */
+    constexpr int SW_STRIDE = S::SW_STRIDE;
+    float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2 tiles][SW_STRIDE]: fp8 [2][D_MAX_KB] weight block scales */
+    int *lds_mtp = reinterpret_cast<int *>(lds_sw + 2 * SW_STRIDE);            /* [experts + 1] tiles of TM rows before expert e */
     int *lds_roff = lds_mtp + (D_MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
     uint16_t *lds_gs = reinterpret_cast<uint16_t *>(lds_roff + (D_MAX_EXPERTS + 1));   /* [NSTAGE][BN] W4A8 group scales (fp16) */
     uint16_t *lds_short = lds_gs + (WRB == 64 ? NSTAGE * BN : 0);                       /* [experts] the short experts, second phase */
@@ -604,27 +611,36 @@ grouped_gemm_dma_kernel(GemmParams p)
      * are clamped onto its last row. 1 KiB block number b = wave + NW*j of the W tile is block b % HALF_BLOCKS of
      * the weight half b / HALF_BLOCKS, a straight copy. Addresses are a wave-uniform base plus a 32-bit lane offset.
      */
-    const int r0 = 8 * wave + (lane >> 3);
-    const uint32_t a_chunk = ((lane & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1))) * 16;
-    const uint32_t w_off = wave * 1024 + lane * 16;
     const uint32_t lds0 = __builtin_amdgcn_readfirstlane(lds_addr(smem) + wave * 1024);     /* this wave's block 0 of stage 0 */
-    const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave % S::ROW_GROUPS) * 256);
-    const bool sa_wave = MODE == MODE_FP8 && wave < S::ROW_GROUPS;
+    constexpr int SA_WAVES = (TM + 63) / 64;          /* waves that bring in 64 activation block scales each */
+    const uint32_t lds_sa0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_sa) + (wave % SA_WAVES) * 256);
+    const bool sa_wave = MODE == MODE_FP8 && wave < SA_WAVES;
     const bool gs_wave = MODE == MODE_W4A8 && wave < 2;            /* wave h brings the group scales of weight half h */
     const uint32_t lds_gs0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_gs) + (wave & 1) * 256);
+    /*
+     * The 288-row shape has no register to spare for the transfers' lane offsets across a K step: there they are worked
+     * out afresh for every transfer from a copy of the lane number that the K loop makes opaque once per step (kept
+     * across the loop they were spilled, and a reload waits for the slabs in flight).
+     */
+    int lane_dma = lane;
     /* part j of a slab: the wave's j-th block of the W tile (j < W_PARTS), of the A tile (j < 4) and, with part 0, the scales */
     auto issue_part = [&](const Tile &t, int kb, int stage, int j) __attribute__((always_inline)) {
+        const int lane_x = TM > 256 ? lane_dma : lane;
+        const int r0 = 8 * wave_u + (lane_x >> 3);
+        const uint32_t a_chunk = ((lane_x & 7) ^ ((r0 & 7) ^ ((r0 >> 3) & 1))) * 16;
+        const uint32_t w_off = wave_u * 1024 + lane_x * 16;
         const uint32_t dst = lds0 + stage * STAGE_BYTES + j * (NW * 1024);
         if (j < W_PARTS) {
             const uint8_t *wsrc = t.w_half[(NW * j) / HALF_BLOCKS] + ((int64_t)kb * W_BLOCK_BYTES + ((NW * j) % HALF_BLOCKS) * 1024);
             if (WSTREAM) dma16_sv_nt(wsrc, w_off, dst + A_BYTES);
             else dma16_sv(wsrc, w_off, dst + A_BYTES);
         }
-        if (j < 4) {
+        if (j < S::A_PARTS && (TM % (8 * NW) == 0 || 8 * NW * j + 8 * wave_u < TM)) {
             /*
              * An 8-row block past the expert's end moves 16 bytes instead of 1 KiB (one lane): the transfer still
              * counts as one operation of this wave, which keeps the outstanding-operation arithmetic the same for
-             * every wave and tile.
+             * every wave and tile. (The 288-row shape waits for all of its transfers every step, so there the blocks
+             * past the tile's 288 rows, the fifth of the upper four waves, are simply not issued.)
              */
             const bool present = 8 * NW * j + 8 * wave_u <= t.last_rel;
             int rel = 8 * NW * j + r0;
@@ -632,12 +648,13 @@ grouped_gemm_dma_kernel(GemmParams p)
             if (present || lane == 0) dma16_sv(t.a_base + (int64_t)kb * BKB, (uint32_t)rel * (uint32_t)K + a_chunk, dst);
         }
         if (j == 0 && sa_wave) {
-            int rel = wave * 64 + lane;
+            int rel = wave_u * 64 + lane_x;
+            const bool in_tile = TM % 64 == 0 || rel < TM;          /* the ring holds TM scales per stage: lanes past that stay out */
             if (rel > t.last_rel) rel = t.last_rel;
-            dma4_sv(t.sa_base + kb, (uint32_t)rel * (uint32_t)KB * 4u, lds_sa0 + stage * TM * 4);
+            if (in_tile) dma4_sv(t.sa_base + kb, (uint32_t)rel * (uint32_t)KB * 4u, lds_sa0 + stage * TM * 4);
         }
         if (j == 0 && gs_wave)      /* 128 fp16 scales = 64 dwords, one per lane */
-            dma4_sv((const float *)(t.gs_mine + (int64_t)kb * p.N), lane * 4u, lds_gs0 + stage * (BN * 2));
+            dma4_sv((const float *)(t.gs_mine + (int64_t)kb * p.N), lane_x * 4u, lds_gs0 + stage * (BN * 2));
     };
     auto issue = [&](const Tile &t, int kb, int stage) __attribute__((always_inline)) {
 #pragma unroll
@@ -652,7 +669,7 @@ grouped_gemm_dma_kernel(GemmParams p)
         for (int b = wave_u * 64; b < KB; b += NW * 64) {
             if (b + lane < KB) {
                 const uint32_t off = (uint32_t)(b + lane) * (uint32_t)sw_stride * 4u;
-                const uint32_t dst = lds_addr(lds_sw) + (buf * 2 * D_MAX_KB + b) * 4;
+                const uint32_t dst = lds_addr(lds_sw) + (buf * SW_STRIDE + b) * 4;
                 dma4_sv(base + c0, off, __builtin_amdgcn_readfirstlane(dst));
                 dma4_sv(base + c1, off, __builtin_amdgcn_readfirstlane(dst) + D_MAX_KB * 4);
             }
@@ -665,8 +682,8 @@ grouped_gemm_dma_kernel(GemmParams p)
      */
     auto issue_es = [&](const Tile &t, int buf) __attribute__((always_inline)) {
         if (MODE != MODE_W8A8) return;
-        const uint32_t dst0 = lds_addr(lds_sw) + buf * 2048;
-        if (wave_u < TM / 64) {
+        const uint32_t dst0 = lds_addr(lds_sw) + buf * SW_STRIDE * 4;
+        if (wave_u < (TM + 63) / 64) {
             int rel = wave_u * 64 + lane;
             if (rel > t.last_rel) rel = t.last_rel;
             dma4_sv(p.a_scale + t.row_begin, (uint32_t)rel * 4u, __builtin_amdgcn_readfirstlane(dst0 + 1024 + wave_u * 256));
@@ -687,7 +704,7 @@ grouped_gemm_dma_kernel(GemmParams p)
         }
     };
     /* this wave's vector-memory operations per slab: what may stay outstanding while an older slab is awaited */
-    constexpr int OPS = W_PARTS + 4;
+    constexpr int OPS = W_PARTS + S::A_PARTS;
     const bool extra_op_wave = sa_wave || gs_wave;                  /* one more operation per slab: the scales */
 
     /* fragment reads: row lane%16 of a 16-row sub-tile, logical chunks 2*(lane/16) and 2*(lane/16)+1 */
@@ -720,10 +737,11 @@ grouped_gemm_dma_kernel(GemmParams p)
         lid = next_id(lid);
         load_tile(lid, nxt);
 
-        f32x4 accf[4][8];
-        i32x4 acci[4][8];
+        constexpr int MTM = S::MTM;
+        f32x4 accf[MTM][8];
+        i32x4 acci[MTM][8];
 #pragma unroll
-        for (int mt = 0; mt < 4; ++mt)
+        for (int mt = 0; mt < MTM; ++mt)
 #pragma unroll
             for (int nt = 0; nt < 8; ++nt) {
                 accf[mt][nt] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -735,8 +753,8 @@ grouped_gemm_dma_kernel(GemmParams p)
          */
         const int tile_subs = (cur.row_end - cur.row_begin + 15) >> 4;
         int mt_act = (tile_subs - wm + RG - 1) / RG;
-        mt_act = mt_act < 0 ? 0 : (mt_act > 4 ? 4 : mt_act);
-        const float *sw_cur = lds_sw + sw_buf * 2 * D_MAX_KB;
+        mt_act = mt_act < 0 ? 0 : (mt_act > MTM ? MTM : mt_act);
+        const float *sw_cur = lds_sw + sw_buf * SW_STRIDE;
 
         /* the K loop over the wave's first MT row sub-tiles; MT is a compile-time constant so that the loops unroll */
         auto k_loop = [&](auto mt_tag) __attribute__((always_inline)) {
@@ -751,6 +769,7 @@ grouped_gemm_dma_kernel(GemmParams p)
                 wait_vmcnt<0>();
             }
             __syncthreads();                /* slab kb has landed for everybody; the stage read in the step before is free */
+            if constexpr (TM > 256) asm volatile("" : "+v"(lane_dma));
             /*
              * The next tile's weight block scales go into the buffer the tile before this one used. Every wave is
              * past this tile's first barrier now, so none of them still reads that buffer; the transfers are older
@@ -780,6 +799,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             auto issue_quarter = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
                 for (int j = q * (PARTS / 4); j < (q + 1) * (PARTS / 4); ++j) issue_part(ft, fill_kb, fill_stage, j);
+                if (PARTS % 4 != 0 && q == 3) issue_part(ft, fill_kb, fill_stage, PARTS - 1);
             };
             auto load_w = [&](int nt) -> i32x8 {
                 const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
@@ -788,10 +808,14 @@ grouped_gemm_dma_kernel(GemmParams p)
             };
 
             if constexpr (MT > 0) {
-                i32x8 af[MT];
+                /* five row sub-tiles in the fp8 mode: two passes over the weight fragments, see below */
+                constexpr bool TWO_PASS = MODE == MODE_FP8 && MT == 5;
+                constexpr bool AF_PER_PASS = TWO_PASS && GMM1;
+                constexpr int AFN = AF_PER_PASS ? 3 : MT;
+                i32x8 af[AFN];
                 i32x8 wf_first = {};
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt) {
+                for (int mt = 0; mt < AFN; ++mt) {
                     const uint8_t *ab = sb + ((RG * mt + wm) * 16) * BKB;
                     const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
                     const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
@@ -815,37 +839,121 @@ grouped_gemm_dma_kernel(GemmParams p)
                      * matrix unit.
                      */
                     const float sw0 = sw_cur[kb], sw1 = sw_cur[D_MAX_KB + kb];
-                    float s0[MT], s1[MT];
+                    if constexpr (MT == 5) {
+                        /*
+                         * Five row sub-tiles: 160 accumulators leave no room for five activation fragments beside the
+                         * weight fragment fetched ahead and the block-scale products. The step goes over the eight
+                         * weight fragments twice, first for row sub-tiles 0-2, then for 3-4, whose activation
+                         * fragments take the registers of the first three (the weight fragments are read again: LDS
+                         * reads are cheap here, registers are not). Each pass is the pipeline of the loop below.
+                         */
+                        auto pass = [&](auto lo_tag, auto n_tag) __attribute__((always_inline)) {
+                            constexpr int M0 = decltype(lo_tag)::value, MN = decltype(n_tag)::value;
+                            constexpr int A0 = AF_PER_PASS ? 0 : M0;       /* where the pass's fragments sit in af */
+                            if constexpr (!AF_PER_PASS) {
+                                /*
+                                 * Second GEMM: a wave's channels share one weight block scale, so one product per row
+                                 * sub-tile does; that leaves room for all five activation fragments from the start, and
+                                 * the weight fragment is read where it is used (measured against the form below on one
+                                 * GPU, 4096 tokens over 32 experts: 0.563 against 0.590 ms; the first GEMM the other way
+                                 * round, 1.16 against 1.00 ms).
+                                 */
+                                const float swx = wn == 1 ? sw1 : sw0;
+                                float sc[MN];
 #pragma unroll
-                    for (int mt = 0; mt < MT; ++mt) {
-                        const float sa = lds_sa[cur_stage * TM + (RG * mt + wm) * 16 + frag_row];
-                        s0[mt] = sa * sw0;
-                        s1[mt] = sa * sw1;
-                    }
-                    i32x8 wf = wf_first;
-                    f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
+                                for (int m = 0; m < MN; ++m)
+                                    sc[m] = lds_sa[cur_stage * TM + (RG * (M0 + m) + wm) * 16 + frag_row] * swx;
 #pragma unroll
-                    for (int nt = 0; nt < 8; ++nt) {
-                        i32x8 wf_n = wf;
-                        if (nt + 1 < 8) wf_n = load_w(nt + 1);
-                        /* the 256-row fp8 loop hands the slab out in two halves (0.6 % faster, measured against quarters on one GPU; the other loops are slower that way) */
-                        if (TM == 256) {
-                            if (more && (nt == 0 || nt == 2)) { issue_quarter(nt); issue_quarter(nt + 1); }
-                        } else if (nt < 4 && more) {
-                            issue_quarter(nt);
-                        }
-                        const bool second = GMM1 ? (nt >= 4) : (wn == 1);
+                                for (int nt = 0; nt < 8; ++nt) {
+                                    const i32x8 wfj = (M0 == 0 && nt == 0) ? wf_first : load_w(nt);
+                                    if (M0 == 0 && more && (nt == 0 || nt == 2)) { issue_quarter(nt); issue_quarter(nt + 1); }
+                                    f32x4 part = mfma_fp8_16x16x128(wfj, af[A0]);
 #pragma unroll
+                                    for (int m = 0; m < MN; ++m) {
+                                        f32x4 nxt_part = part;
+                                        if (m + 1 < MN) nxt_part = mfma_fp8_16x16x128(wfj, af[A0 + m + 1]);
+#pragma unroll
+                                        for (int i = 0; i < 4; ++i) accf[M0 + m][nt][i] = __builtin_fmaf(part[i], sc[m], accf[M0 + m][nt][i]);
+                                        part = nxt_part;
+                                    }
+                                }
+                                return;
+                            }
+                            i32x8 wf = wf_first;
+                            if (M0 != 0) {
+                                asm volatile("" ::: "memory");        /* not before the first pass is through with af */
+#pragma unroll
+                                for (int m = 0; m < MN; ++m) {
+                                    const uint8_t *ab = sb + ((RG * (M0 + m) + wm) * 16) * BKB;
+                                    const u32x4 lo = *reinterpret_cast<const u32x4 *>(ab + off_lo);
+                                    const u32x4 hi = *reinterpret_cast<const u32x4 *>(ab + off_hi);
+                                    af[m] = i32x8{(int)lo[0], (int)lo[1], (int)lo[2], (int)lo[3], (int)hi[0], (int)hi[1], (int)hi[2], (int)hi[3]};
+                                    if (m == 0) wf = load_w(0);
+                                }
+                            }
+                            float s0[MN], s1[MN];
+#pragma unroll
+                            for (int m = 0; m < MN; ++m) {
+                                const float sa = lds_sa[cur_stage * TM + (RG * (M0 + m) + wm) * 16 + frag_row];
+                                s0[m] = sa * sw0;
+                                s1[m] = sa * sw1;
+                            }
+                            f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
+#pragma unroll
+                            for (int nt = 0; nt < 8; ++nt) {
+                                i32x8 wf_n = wf;
+                                if (nt + 1 < 8) wf_n = load_w(nt + 1);
+                                if (M0 == 0 && more && (nt == 0 || nt == 2)) { issue_quarter(nt); issue_quarter(nt + 1); }
+                                const bool second = GMM1 ? (nt >= 4) : (wn == 1);
+#pragma unroll
+                                for (int m = 0; m < MN; ++m) {
+                                    f32x4 nxt_part = part;
+                                    if (m + 1 < MN) nxt_part = mfma_fp8_16x16x128(wf, af[m + 1]);
+                                    else if (nt + 1 < 8) nxt_part = mfma_fp8_16x16x128(wf_n, af[0]);
+                                    const float sc = second ? s1[m] : s0[m];
+#pragma unroll
+                                    for (int i = 0; i < 4; ++i) accf[M0 + m][nt][i] = __builtin_fmaf(part[i], sc, accf[M0 + m][nt][i]);
+                                    part = nxt_part;
+                                }
+                                wf = wf_n;
+                            }
+                        };
+                        pass(std::integral_constant<int, 0>{}, std::integral_constant<int, 3>{});
+                        pass(std::integral_constant<int, 3>{}, std::integral_constant<int, 2>{});
+                    } else {
+
+                        float s0[MT], s1[MT];
+    #pragma unroll
                         for (int mt = 0; mt < MT; ++mt) {
-                            f32x4 nxt_part = part;
-                            if (mt + 1 < MT) nxt_part = mfma_fp8_16x16x128(wf, af[mt + 1]);
-                            else if (nt + 1 < 8) nxt_part = mfma_fp8_16x16x128(wf_n, af[0]);
-                            const float sc = second ? s1[mt] : s0[mt];
-#pragma unroll
-                            for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
-                            part = nxt_part;
+                            const float sa = lds_sa[cur_stage * TM + (RG * mt + wm) * 16 + frag_row];
+                            s0[mt] = sa * sw0;
+                            s1[mt] = sa * sw1;
                         }
-                        wf = wf_n;
+                        i32x8 wf = wf_first;
+                        f32x4 part = mfma_fp8_16x16x128(wf, af[0]);
+    #pragma unroll
+                        for (int nt = 0; nt < 8; ++nt) {
+                            i32x8 wf_n = wf;
+                            if (nt + 1 < 8) wf_n = load_w(nt + 1);
+                            /* the 256-row fp8 loop hands the slab out in two halves (0.6 % faster, measured against quarters on one GPU; the other loops are slower that way) */
+                            if (TM == 256) {
+                                if (more && (nt == 0 || nt == 2)) { issue_quarter(nt); issue_quarter(nt + 1); }
+                            } else if (nt < 4 && more) {
+                                issue_quarter(nt);
+                            }
+                            const bool second = GMM1 ? (nt >= 4) : (wn == 1);
+    #pragma unroll
+                            for (int mt = 0; mt < MT; ++mt) {
+                                f32x4 nxt_part = part;
+                                if (mt + 1 < MT) nxt_part = mfma_fp8_16x16x128(wf, af[mt + 1]);
+                                else if (nt + 1 < 8) nxt_part = mfma_fp8_16x16x128(wf_n, af[0]);
+                                const float sc = second ? s1[mt] : s0[mt];
+    #pragma unroll
+                                for (int i = 0; i < 4; ++i) accf[mt][nt][i] = __builtin_fmaf(part[i], sc, accf[mt][nt][i]);
+                                part = nxt_part;
+                            }
+                            wf = wf_n;
+                        }
                     }
                 } else if constexpr (MODE == MODE_W4A8) {
                     /*
@@ -924,14 +1032,15 @@ grouped_gemm_dma_kernel(GemmParams p)
             }
         }
         };
-        if (mt_act == 4) k_loop(std::integral_constant<int, 4>{});
+        if (MTM == 5 && mt_act == 5) k_loop(std::integral_constant<int, MTM == 5 ? 5 : 4>{});
+        else if (mt_act == 4) k_loop(std::integral_constant<int, 4>{});
         else if (mt_act == 3) k_loop(std::integral_constant<int, 3>{});
         else if (mt_act == 2) k_loop(std::integral_constant<int, 2>{});
         else if (mt_act == 1) k_loop(std::integral_constant<int, 1>{});
         else k_loop(std::integral_constant<int, 0>{});
         if constexpr (MODE == MODE_W4A8) {      /* the unpacked weights were 16 x their value; a power of two divides out exactly */
 #pragma unroll
-            for (int mt = 0; mt < 4; ++mt)
+            for (int mt = 0; mt < MTM; ++mt)
 #pragma unroll
                 for (int nt = 0; nt < 8; ++nt)
 #pragma unroll
@@ -948,8 +1057,8 @@ grouped_gemm_dma_kernel(GemmParams p)
          */
         int lane_e = lane;
         asm volatile("" : "+v"(lane_e));
-        epilogue<MODE, GMM1, OUT_DT, RG>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane_e, lds_rowmax, TM,
-                                         lds_sw + sw_buf * 512);
+        epilogue<MODE, GMM1, OUT_DT, RG, S::MTM>(p, tc, accf, acci, cur.row_begin, cur.row_end, wm, wn, lane_e, lds_rowmax, TM,
+                                         lds_sw + sw_buf * SW_STRIDE);
         if (!nxt.valid) break;
         cur = nxt;
         sw_buf ^= 1;
@@ -1045,6 +1154,8 @@ int32_t prepare_mode()
 {
     int n = 0;
     int32_t rc = prepare_shape<MODE, GMM1, OUT_DT, 256, 2, false>(nullptr, &n);
+    if constexpr (MODE != MODE_W4A8)
+        if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 288, 2, false>(nullptr, &n);
     if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 128, 3, false>(nullptr, &n);
     if constexpr (MODE != MODE_W4A8)
         if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 128, 3, true>(nullptr, &n);
@@ -1054,14 +1165,14 @@ int32_t prepare_mode()
 /*
  * Shape choice from what the host knows (the row counts themselves live on the device). With few rows per expert the
  * GEMM is a weight-streaming job and takes the three-stage 128-row shape (which needs two K slabs to fill its
- * pipeline); with many it needs the arithmetic intensity of the 256-row shape. Where the two meet was measured on
- * 7168 x 4096 / 2048 x 7168 experts (W4A8: 4096 x 3072), rows per expert on average:
- *   - few tiles (experts x channel tiles <= 1024, e.g. 32 experts): the small tiles also balance the CUs better, and
- *     the 128-row shape stays ahead up to 384 rows (W8A8: 15 % at 256 rows, 4 % at 384, behind by 1 % at 512) and up
- *     to 256 rows in the first fp8 GEMM (10 % at 160-192 rows, equal at 256);
- *   - many tiles (128 or 256 experts): the shapes meet between 96 and 128 rows for fp8 (256 experts, 128 rows: the
- *     256-row shape 6 % ahead; 96 rows: 9 % behind), and at 128-192 rows for W8A8;
- *   - the second fp8 GEMM (16 K slabs per tile, bf16 rows out) prefers the 256-row shape from 128 rows on in both cases;
+ * pipeline); with many it needs the arithmetic intensity of a two-stage shape, 288 or 256 rows high. All three were
+ * timed on 7168 x 4096 / 2048 x 7168 experts (W4A8: 4096 x 3072) with 32 and with 256 experts, random routing, rows
+ * per expert on average:
+ *   - fp8: the 128-row shape stays ahead up to 96 rows in both GEMMs (32 experts, first GEMM: 0.216 against 0.242 ms
+ *     at 96 rows, 0.283 against 0.253 at 128; 256 experts: 1.56 against 1.76 at 96, 2.24 against 1.88 at 128);
+ *   - W8A8, first GEMM: equal at 128 rows (0.254 / 0.255 ms; 256 experts 1.846 / 1.854), the tall shape 9 % ahead at
+ *     192; second GEMM (16 K slabs per tile): the 128-row shape 5-12 % ahead at 128 rows, equal at 192 with 32 experts
+ *     and 13 % behind there with 256;
  *   - W4A8's few-row kernel is bound by the unpack and promote instructions of its one wave per SIMD, not by the
  *     weight stream: equal at 64 rows, the 256-row shape 2 % ahead at 96 and 17 % at 128 (a fourth stage for the
  *     half-size packed slabs changed nothing).
@@ -1070,11 +1181,24 @@ template <int MODE, bool GMM1>
 inline int64_t few_rows_limit(const GemmParams &p, int n_tiles)
 {
     if (MODE == MODE_W4A8) return 64;
+    if (MODE == MODE_FP8) return 96;
+    if (GMM1) return 128;
     const bool few_tiles = (int64_t)p.experts * n_tiles <= 1024;
-    if (MODE == MODE_W8A8) return few_tiles ? 384 : 128;
-    if (GMM1) return few_tiles ? 256 : 96;
-    return 96;
+    return few_tiles ? 192 : 128;
 }
+
+/*
+ * Two thirds of a two-stage tile's time does not depend on its rows (weight fragments, barrier, slab transfers), so
+ * the fewer row tiles an expert has the better, and an expert whose rows just miss a multiple of 256 pays for a whole
+ * tile more. The 288-row shape cuts an expert into ceil(rows / 288) even tiles: where that is as many as
+ * ceil(rows / 256) they are the same tiles as the 256-row shape's (and cost 1-4 % more in this kernel), where it is one
+ * less the expert is a tile's fixed cost shorter. Under random routing the second case is common as long as an expert
+ * has few tiles. Measured against the 256-row shape, first / second GEMM, rows per expert on average: fp8 256 rows
+ * -29 % / -15 %, 512 rows -16 % / -9 %, 1024 rows -7.6 % / -4.7 %, 1500 rows -2 % / +1.4 %, 2048 rows +0.5 % / +2 %;
+ * W8A8 256 rows -26 % / -17 %, 1024 rows -7 % / -7 %; with exactly 1024 rows for every expert fp8 +3 % / +4.6 %.
+ * W4A8 has no such shape (its loop has no registers for a fifth row sub-tile).
+ */
+constexpr int64_t kTallRowsLimit = 1536;
 
 template <int MODE, bool GMM1, int OUT_DT>
 int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
@@ -1092,6 +1216,9 @@ int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
             if ((int64_t)p.max_rows <= stream_limit * (int64_t)p.experts) return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3, true>(p, n_tiles, st);
         }
         return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
+    }
+    if constexpr (MODE != MODE_W4A8) {
+        if ((int64_t)p.max_rows <= kTallRowsLimit * (int64_t)p.experts) return launch_dma_shape<MODE, GMM1, OUT_DT, 288, 2>(p, n_tiles, st);
     }
     return launch_dma_shape<MODE, GMM1, OUT_DT, 256, 2>(p, n_tiles, st);
 }
