@@ -255,7 +255,8 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
 
 /* ------------------------------------------------------------------------------------------------------
  * The grouped GEMM kernel (W8A8, fp8, W4A8): TM token rows x 256 channels x 128 K elements per workgroup,
- * TM/64 x 2 waves with a 64 x 128 wave tile each, one workgroup per CU.
+ * eight waves (four row groups x two 128-channel halves; a wave's rows are the 16-row sub-tiles s with
+ * s % 4 = its row group), one workgroup per CU.
  *
  * K slabs go from HBM to LDS without passing through registers: every wave issues
  * global_load_lds_dwordx4, which deposits the 64 lanes' 16-byte chunks in 1 KiB of consecutive LDS
@@ -266,10 +267,11 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
  * pairs, so the read is free of bank conflicts whether the LDS serves 8 or 16 lanes per pass; plain
  * row-major storage would put all 16 rows on the same slot.
  *
- * Two shapes are built. TM = 256 with two stages of 64 KiB (the slab for step k+1 is in flight while step k
- * is multiplied) has the arithmetic intensity that many-row experts need. TM = 128 with three stages of
- * 48 KiB is for few-row experts, where the job is to stream every weight byte once at HBM speed: it keeps
- * two weight slabs (64 KiB) in flight per CU and skips the MFMAs of 16-row groups past the expert's end.
+ * Three shapes are built. TM = 256 and TM = 288 with two stages of 64 / 68 KiB (the slab for step k+1 is in
+ * flight while step k is multiplied) have the arithmetic intensity that many-row experts need; the 288-row
+ * shape gives the waves of two row groups a fifth sub-tile. TM = 128 with three stages of 48 KiB is for
+ * few-row experts, where the job is to stream every weight byte once at HBM speed: it keeps two weight slabs
+ * (64 KiB) in flight per CU, two sub-tiles per wave, and skips the MFMAs of sub-tiles past the expert's end.
  * Either way there is one barrier per step.
  *
  * W4A8: the weight slab stays packed in LDS (64 bytes per channel; block layout and nibble order as written by
@@ -283,7 +285,7 @@ constexpr int D_MAX_EXPERTS = 1024;
 /* WRB = bytes of one weight row per slab: 128 (8-bit) or 64 (packed int4) */
 template <int TM, int NSTAGE, int WRB>
 struct DmaShape {
-    static constexpr int ROW_GROUPS = TM > 256 ? 4 : TM / 64;
+    static constexpr int ROW_GROUPS = 4;                   /* row groups of two waves each: eight waves, two per SIMD */
     static constexpr int MTM = (TM / 16 + ROW_GROUPS - 1) / ROW_GROUPS;   /* 16-row sub-tiles per wave, at most: 4, or 5 in the 288-row shape */
     static constexpr int NW = ROW_GROUPS * 2;
     static constexpr int THREADS = NW * 64;
@@ -302,8 +304,8 @@ struct DmaShape {
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + SW_BYTES +
                                      2 * (D_MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0) +
                                      (TWO_PHASE ? D_MAX_EXPERTS * 2 + (D_MAX_EXPERTS + 1) * 4 : 0);
-    static_assert((A_PARTS == 4 && PARTS % 4 == 0) || (TM == 288 && NSTAGE == 2 && PARTS == 5),
-                  "the issue schedule hands out a slab in four quarters (the 288-row shape: a fifth part with the last quarter)");
+    static_assert(PARTS >= 2 && (PARTS % 4 == 0 || PARTS == 2 || (NSTAGE == 2 && PARTS == 5)),
+                  "the issue schedule hands out parts q * PARTS / 4 .. (q + 1) * PARTS / 4 - 1 of a slab with quarter q of a step");
     static_assert(NW <= HALF_BLOCKS && HALF_BLOCKS % NW == 0, "a wave's W blocks must not straddle a weight half");
     static_assert(LDS_BYTES <= 160 * 1024, "tile does not fit the LDS");
 };
@@ -384,13 +386,12 @@ struct DmaTile {
 
 template <int MODE, bool GMM1, int OUT_DT, int TM, int NSTAGE, bool WSTREAM>
 /*
- * TM/64 x 2 waves. The second bound is waves per SIMD, i.e. the register budget: 256 registers with two waves, 512 with
- * one. The 128-row shape has one wave per SIMD anyway; its fp8 flavour needs more than 256 registers (block-scale
- * products beside the accumulators) and with 256 it spilled inside the K loop, where a scratch reload also waits for
- * the slabs in flight (1.7x slower than the 256-row shape on few-row experts). The int flavours fit 256 and are
- * a little faster compiled for it.
+ * Eight waves, two per SIMD (256 registers each), in every shape. The 128-row shape used to run four waves with the
+ * wave tile of the 256-row shape (64 x 128), one per SIMD with nobody to cover its waits; as eight waves of 32 x 128
+ * it is faster wherever it is used: decode layer (128 tokens, W8A8) 0.295 -> 0.288 ms, fp8 with 96 rows per expert
+ * on 32 experts 0.404 -> 0.342 ms, W4A8 with 32-96 rows per expert first GEMM 9-12 % and second 7-8 % faster.
  */
-__global__ void __launch_bounds__(TM > 256 ? 512 : TM * 2, (TM == 128 && MODE == MODE_FP8) ? 1 : 2)
+__global__ void __launch_bounds__(512, 2)
 grouped_gemm_dma_kernel(GemmParams p)
 {
     static_assert(MODE == MODE_W8A8 || MODE == MODE_FP8 || MODE == MODE_W4A8, "unknown mode");
@@ -798,8 +799,7 @@ grouped_gemm_dma_kernel(GemmParams p)
             }
             auto issue_quarter = [&](int q) __attribute__((always_inline)) {
 #pragma unroll
-                for (int j = q * (PARTS / 4); j < (q + 1) * (PARTS / 4); ++j) issue_part(ft, fill_kb, fill_stage, j);
-                if (PARTS % 4 != 0 && q == 3) issue_part(ft, fill_kb, fill_stage, PARTS - 1);
+                for (int j = q * PARTS / 4; j < (q + 1) * PARTS / 4; ++j) issue_part(ft, fill_kb, fill_stage, j);
             };
             auto load_w = [&](int nt) -> i32x8 {
                 const u32x4 lo = *reinterpret_cast<const u32x4 *>(sb + w_sub[nt] + off_lo);
@@ -1003,20 +1003,12 @@ grouped_gemm_dma_kernel(GemmParams p)
                 } else {
                     /*
                      * int8: lane's 32 K bytes feed two 64-deep MFMAs; the two updates of one accumulator are kept apart.
-                     * The 128-row shape has one wave per SIMD and nobody to cover an LDS read's latency, so it asks for
-                     * the next weight fragment before the MFMAs of this one (1024 tokens over 32 experts: GMM1 2.5 %
-                     * faster, decode 0.4 %); with two waves per SIMD the same order was 0.5 % slower.
+                     * (Asking for the next weight fragment before the MFMAs of this one was 0.5 % slower here: the
+                     * SIMD's other wave covers the read.)
                      */
-                    i32x8 wf_ahead = wf_first;
 #pragma unroll
                     for (int nt = 0; nt < 8; ++nt) {
-                        i32x8 wf;
-                        if (TM == 128) {
-                            wf = wf_ahead;
-                            if (nt + 1 < 8) wf_ahead = load_w(nt + 1);
-                        } else {
-                            wf = nt == 0 ? wf_first : load_w(nt);
-                        }
+                        const i32x8 wf = nt == 0 ? wf_first : load_w(nt);
                         if (nt < 4 && more) issue_quarter(nt);
                         const i32x4 wf0 = i32x4{wf[0], wf[1], wf[2], wf[3]}, wf1 = i32x4{wf[4], wf[5], wf[6], wf[7]};
 #pragma unroll
@@ -1032,10 +1024,10 @@ grouped_gemm_dma_kernel(GemmParams p)
             }
         }
         };
-        if (MTM == 5 && mt_act == 5) k_loop(std::integral_constant<int, MTM == 5 ? 5 : 4>{});
-        else if (mt_act == 4) k_loop(std::integral_constant<int, 4>{});
-        else if (mt_act == 3) k_loop(std::integral_constant<int, 3>{});
-        else if (mt_act == 2) k_loop(std::integral_constant<int, 2>{});
+        if (MTM >= 5 && mt_act == 5) k_loop(std::integral_constant<int, MTM >= 5 ? 5 : MTM>{});
+        else if (MTM >= 4 && mt_act == 4) k_loop(std::integral_constant<int, MTM >= 4 ? 4 : MTM>{});
+        else if (MTM >= 3 && mt_act == 3) k_loop(std::integral_constant<int, MTM >= 3 ? 3 : MTM>{});
+        else if (MTM >= 2 && mt_act == 2) k_loop(std::integral_constant<int, MTM >= 2 ? 2 : MTM>{});
         else if (mt_act == 1) k_loop(std::integral_constant<int, 1>{});
         else k_loop(std::integral_constant<int, 0>{});
         if constexpr (MODE == MODE_W4A8) {      /* the unpacked weights were 16 x their value; a power of two divides out exactly */
@@ -1165,26 +1157,25 @@ int32_t prepare_mode()
 /*
  * Shape choice from what the host knows (the row counts themselves live on the device). With few rows per expert the
  * GEMM is a weight-streaming job and takes the three-stage 128-row shape (which needs two K slabs to fill its
- * pipeline); with many it needs the arithmetic intensity of a two-stage shape, 288 or 256 rows high. All three were
- * timed on 7168 x 4096 / 2048 x 7168 experts (W4A8: 4096 x 3072) with 32 and with 256 experts, random routing, rows
- * per expert on average:
- *   - fp8: the 128-row shape stays ahead up to 96 rows in both GEMMs (32 experts, first GEMM: 0.216 against 0.242 ms
- *     at 96 rows, 0.283 against 0.253 at 128; 256 experts: 1.56 against 1.76 at 96, 2.24 against 1.88 at 128);
- *   - W8A8, first GEMM: equal at 128 rows (0.254 / 0.255 ms; 256 experts 1.846 / 1.854), the tall shape 9 % ahead at
- *     192; second GEMM (16 K slabs per tile): the 128-row shape 5-12 % ahead at 128 rows, equal at 192 with 32 experts
- *     and 13 % behind there with 256;
- *   - W4A8's few-row kernel is bound by the unpack and promote instructions of its one wave per SIMD, not by the
- *     weight stream: equal at 64 rows, the 256-row shape 2 % ahead at 96 and 17 % at 128 (a fourth stage for the
- *     half-size packed slabs changed nothing).
+ * pipeline); with many it needs the arithmetic intensity of a two-stage shape, 288 or 256 rows high. The shapes were
+ * timed against each other on 7168 x 4096 / 2048 x 7168 experts (W4A8: 4096 x 3072 / 1536 x 4096, 128 experts) with 32
+ * and with 256 experts, random routing; rows per expert on average, first / second GEMM, 128-row against 288-row
+ * (W4A8: 256-row) shape in ms:
+ *   - fp8, 32 experts: 128 rows 0.247 / 0.136 against 0.256 / 0.145; 192 rows 0.298 / 0.160 against 0.278 / 0.166;
+ *     256 rows 0.369 / 0.194 against 0.306 / 0.188. 256 experts: 128 rows 1.889 / 0.961 against 1.877 / 1.088;
+ *     192 rows 2.314 / 1.204 against 2.108 / 1.148;
+ *   - W8A8, 32 experts: 128 rows 0.243 / 0.129 against 0.254 / 0.138; 192 rows 0.289 / 0.146 against 0.275 / 0.150;
+ *     256 rows 0.342 / 0.174 against 0.303 / 0.163. 256 experts: 128 rows 1.788 / 0.892 against 1.799 / 0.931;
+ *     192 rows 2.197 / 1.093 against 2.016 / 1.106;
+ *   - W4A8: 96 rows 0.358 / 0.171 against 0.366 / 0.178; 128 rows 0.503 / 0.237 against 0.457 / 0.216.
  */
 template <int MODE, bool GMM1>
 inline int64_t few_rows_limit(const GemmParams &p, int n_tiles)
 {
-    if (MODE == MODE_W4A8) return 64;
-    if (MODE == MODE_FP8) return 96;
+    if (MODE == MODE_W4A8) return 96;
     if (GMM1) return 128;
     const bool few_tiles = (int64_t)p.experts * n_tiles <= 1024;
-    return few_tiles ? 192 : 128;
+    return (MODE == MODE_FP8 && !few_tiles) ? 128 : 192;
 }
 
 /*

@@ -303,8 +303,9 @@ def test_gmm1_fp8_many_tiles_per_workgroup(buf, E, K, N1, rows):
 
 # ---- W4A8 ----------------------------------------------------------------------------------------------------------
 
-# 64 rows per expert is the last size that takes the 128-row shape in this mode
-@pytest.mark.parametrize("E,K,N,rows", [(4, 256, 256, 300), (16, 1024, 512, 200), (4, 256, 256, 256), (4, 256, 256, 260)])
+# 96 rows per expert is the last size that takes the 128-row shape in this mode
+@pytest.mark.parametrize("E,K,N,rows", [(4, 256, 256, 300), (16, 1024, 512, 200), (4, 256, 256, 384), (4, 256, 256, 388),
+                                        (2, 256, 512, 700)])
 def test_w4a8_bit_exact(buf, E, K, N, rows):
     counts = ragged_counts(E, rows, E + K)
     a = rng(41).integers(-127, 128, (rows, K)).astype(np.int8)
