@@ -41,10 +41,19 @@ if ROOT not in sys.path:
 
 PEAK_FP8_TFLOPS = 5000.0      # MI355X dense fp8 MFMA
 PEAK_HBM_GBS = 8000.0         # MI355X HBM3E
-# HBM bytes one GMM1 launch moves at the headline workload: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from two
-# `rocprofv3 --pmc` runs of this script (summary and counter calibration: profiles/moe_prefill_fp8_kernels.txt)
-GMM1_TRAFFIC_BYTES_T4096 = 2.29e9
-REDUCE_TRAFFIC_BYTES = 2.416e9  # 2.0 x 1048607 KiB + 262144 KiB (profiles/reduce_8x256MiB.txt)
+
+
+def measured_traffic(key):
+    """HBM bytes per launch of the dominant kernel of workload `key`, or None: 2.0 x FETCH_SIZE + 1.0 x WRITE_SIZE from
+    two `rocprofv3 --pmc` runs of this script, written to profiles/traffic.json together with the profile summaries
+    that show the counters and their calibration (the file names the summary of every entry)."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "traffic.json")) as f:
+            entry = json.load(f).get(key)
+        return None if entry is None else float(entry["bytes_per_launch"])
+    except (OSError, ValueError, KeyError, TypeError):
+        return None
+
 
 
 def parse():
@@ -54,9 +63,10 @@ def parse():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--tokens", type=int, default=4096, help="development only; the reported workload is 4096")
     ap.add_argument("--cpu-sample-tokens", type=int, default=2560)
-    ap.add_argument("--workload", choices=["prefill", "decode", "qwen_w4a8", "reduce"], default="prefill",
-                    help="prefill = the headline fp8 MoE layer (default); decode = 128-token W8A8 layer with Zipf routing; "
-                         "qwen_w4a8 = 16384-token W4A8 layer; reduce = the 8 x 256 MiB local reduction")
+    ap.add_argument("--workload", choices=["prefill", "prefill_w8a8", "decode", "qwen_w4a8", "reduce"], default="prefill",
+                    help="prefill = the headline fp8 MoE layer (default); prefill_w8a8 = the same shape in W8A8 (profiling: no "
+                         "BASELINE configuration); decode = 128-token W8A8 layer with Zipf routing; qwen_w4a8 = 16384-token "
+                         "W4A8 layer; reduce = the 8 x 256 MiB local reduction")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--equal-rows", action="store_true",
                     help="profiling only (prefill): token t picks experts (t*topk + j) mod experts, so every expert receives "
@@ -120,6 +130,9 @@ def other_workloads(args, torch, np, capi, buf):
 MOE_WORKLOADS = {
     "prefill": dict(name="DeepSeek-V3-style prefill share (BASELINE configs[1])", T=4096, H=7168, E=32, K=8, I=2048,
                     mode=2, zipf=None, quant="fp8 e4m3, act 1x128, weight 128x128", dtype="fp8_e4m3"),
+    "prefill_w8a8": dict(name="the prefill share's shape in W8A8 (profiling; not a BASELINE configuration)", T=4096, H=7168, E=32,
+                         K=8, I=2048, mode=1, zipf=None, quant="W8A8 int8, per-token act, per-channel weight scales",
+                         dtype="int8"),
     "decode": dict(name="low-latency decode share (BASELINE configs[2])", T=128, H=7168, E=32, K=8, I=2048,
                    mode=1, zipf=1.2, quant="W8A8 int8, per-token act, per-channel weight scales", dtype="int8"),
     "qwen_w4a8": dict(name="Qwen3-MoE-style W4A8 layer (BASELINE configs[4])", T=16384, H=4096, E=128, K=8, I=1536,
@@ -266,11 +279,12 @@ def bench_moe(args, torch, np, capi, buf, workload):
                     "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": wbytes1 / t1 / 1e9 / PEAK_HBM_GBS, "traffic": None,
                     "experts_with_tokens": touched}
     else:
-        kname = "grouped_gemm_dma_kernel<fp8, gmm1>" if mode == 2 else "grouped_gemm_dma_kernel<w4a8, gmm1>"
+        kname = "grouped_gemm_dma_kernel<%s, gmm1>" % {1: "int8", 2: "fp8", 3: "w4a8"}[mode]
+        routed = workload in ("prefill", "qwen_w4a8") and T == cfg["T"] and not args.equal_rows
         roofline = {"kernel": kname, "bound": "mfma", "achieved": flops1 / t1 / 1e12,
                     "peak": PEAK_FP8_TFLOPS, "unit": "TFLOP/s" if mode == 2 else "TOP/s",
                     "frac": flops1 / t1 / 1e12 / PEAK_FP8_TFLOPS,
-                    "traffic": GMM1_TRAFFIC_BYTES_T4096 if (workload == "prefill" and T == 4096 and not args.equal_rows) else None}
+                    "traffic": measured_traffic(workload + "_gmm1") if routed else None}
     stages = {
         "ms": {k: round(v, 4) for k, v in stage_ms.items()},
         "gmm1_tflops": flops1 / t1 / 1e12,
@@ -376,7 +390,7 @@ def bench_reduce(args, torch, np, capi, buf):
             "config": {"workload": "local reduce-scatter shard (BASELINE configs[3])", "buffers": R,
                        "bytes_per_buffer": nbytes},
             "roofline": {"kernel": "reduce_kernel<bf16, sum, 8>", "bound": "hbm", "achieved": b["gbs"], "peak": PEAK_HBM_GBS,
-                         "unit": "GB/s", "frac": b["gbs"] / PEAK_HBM_GBS, "traffic": REDUCE_TRAFFIC_BYTES},
+                         "unit": "GB/s", "frac": b["gbs"] / PEAK_HBM_GBS, "traffic": measured_traffic("reduce_8x256MiB_bf16")},
             "cpu_baseline": None, "variants": results}
     return line
 

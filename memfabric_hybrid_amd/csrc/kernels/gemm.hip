@@ -640,13 +640,13 @@ grouped_gemm_dma_kernel(GemmParams p)
             /*
              * An 8-row block past the expert's end moves 16 bytes instead of 1 KiB (one lane): the transfer still
              * counts as one operation of this wave, which keeps the outstanding-operation arithmetic the same for
-             * every wave and tile. (The 288-row shape waits for all of its transfers every step, so there the blocks
-             * past the tile's 288 rows, the fifth of the upper four waves, are simply not issued.)
+             * every wave and tile. (The two-stage shapes wait for all of their transfers every step, so there a block
+             * past the tile's end is simply not issued.)
              */
             const bool present = 8 * NW * j + 8 * wave_u <= t.last_rel;
             int rel = 8 * NW * j + r0;
             if (rel > t.last_rel) rel = t.last_rel;
-            if (present || lane == 0) dma16_sv(t.a_base + (int64_t)kb * BKB, (uint32_t)rel * (uint32_t)K + a_chunk, dst);
+            if ((present || lane == 0) && (present || NSTAGE != 2)) dma16_sv(t.a_base + (int64_t)kb * BKB, (uint32_t)rel * (uint32_t)K + a_chunk, dst);
         }
         if (j == 0 && sa_wave) {
             int rel = wave_u * 64 + lane_x;
