@@ -120,6 +120,15 @@ void RemoveUsr1()
         sem_destroy(&gDumpRequests);
     }
 }
+
+/*
+ * A process may end (or unload the library) without calling unbootstrap: the helper thread is then still waiting, and
+ * a std::thread destroyed while joinable ends the process with std::terminate. This object is defined after the
+ * thread, so it is destroyed first and takes the thread down the ordinary way.
+ */
+struct DumpThreadAtExit {
+    ~DumpThreadAtExit() { RemoveUsr1(); }
+} gDumpThreadAtExit;
 } // namespace
 
 /* the kernel launchers' way to leave a last-error text (declared in kernels/zbal_device.h) */

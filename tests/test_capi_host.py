@@ -314,6 +314,24 @@ def test_sigusr1_is_deferred_chained_and_restored(lib):
         signal.signal(signal.SIGUSR1, before)
 
 
+def test_a_process_that_ends_without_unbootstrap_exits_cleanly():
+    """The helper thread that bootstrap starts is taken down when the library's statics go: a process that never calls
+    zbal_unbootstrap must still end with its own exit code (a joinable std::thread destroyed at exit would abort)."""
+    import subprocess
+    import sys
+    code = ("import ctypes\n"
+            "from memfabric_hybrid_amd import capi\n"
+            "lib = capi.load()\n"
+            "opts = capi.BootstrapOptions()\n"
+            "assert lib.zbal_bootstrap_options_init(ctypes.byref(opts)) == 0\n"
+            "opts.flags = 1\n"
+            "assert lib.zbal_bootstrap(ctypes.byref(opts), None) == 0\n"
+            "raise SystemExit(7)\n")
+    done = subprocess.run([sys.executable, "-c", code], cwd=os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                          capture_output=True, text=True, timeout=120)
+    assert done.returncode == 7, (done.returncode, done.stderr[-400:])
+
+
 def test_deepep_buffer_signatures_follow_the_reference():
     """Parameter names, order and defaults of the DeepEP-compatible Buffer, as the reference's Python face declares
     them (app/zbal/src/python/zbal/zbal_buffer.py:28-37, 168-175, 216-232, 350-360, 432-443, 536-545, 611-634)."""
