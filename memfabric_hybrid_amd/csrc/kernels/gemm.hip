@@ -1197,13 +1197,14 @@ int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
     if ((int64_t)p.max_rows <= few_rows_limit<MODE, GMM1>(p, n_tiles) * (int64_t)p.experts && p.K >= 256) {
         /*
          * With few rows per expert nearly every expert has a single row tile and its weight slabs are read once: they
-         * are requested with the streaming hint. Measured: at 32 rows per expert on average 2.5-8 % faster in both
-         * modes (32 and 256 experts, uniform and Zipf routing); at 64 rows W8A8 2.5 % faster, fp8 1-4 % slower; at 128
-         * rows and more, where row tiles share slabs through the L2, 4-7 % slower. W4A8's few-row kernel is not bound
-         * by the stream and stays as it is.
+         * are requested with the streaming hint. Measured on 32 experts of 7168 x 4096 / 2048 x 7168, first / second
+         * GEMM: at 32 rows per expert on average fp8 11 % / 2 % and W8A8 7 % / 6 % faster (decode layer, Zipf routing:
+         * 0.304 -> 0.288 ms); at 64 rows W8A8 4.5 % / 2 % faster, fp8 equal; at 96 rows W8A8 3 % / 0 % faster, fp8
+         * 4 % / 1 % slower; at 128 rows, where row tiles share slabs through the L2, both 5-9 % slower. W4A8's few-row
+         * kernel is bound by its unpack and promote instructions: 1-2 % with the hint at 32-96 rows, left as it is.
          */
         if constexpr (MODE != MODE_W4A8) {
-            const int64_t stream_limit = MODE == MODE_W8A8 ? 64 : 32;
+            const int64_t stream_limit = MODE == MODE_W8A8 ? 96 : 32;
             if ((int64_t)p.max_rows <= stream_limit * (int64_t)p.experts) return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3, true>(p, n_tiles, st);
         }
         return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
