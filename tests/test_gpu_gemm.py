@@ -763,7 +763,8 @@ def test_w8a8_gemms_random_row_counts_bit_exact(buf, seed):
             hot = r.choice(E, size=min(E, 3), replace=False)
             counts[hot] = r.integers(1, 1500, size=len(hot))
         elif style == 2:
-            counts = r.choice([0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 383, 384, 385, 513], size=E)
+            counts = r.choice([0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 271, 272, 273, 287, 288, 289, 383, 384,
+                               385, 513, 575, 576, 577], size=E)
             if counts.sum() > 6000:
                 counts = counts // 4
         else:
