@@ -1057,22 +1057,41 @@ grouped_gemm_dma_kernel(GemmParams p)
     }
 }
 
-/* second pass of the int8 GMM1 epilogue: whole-row requantisation from the fp32 SwiGLU values */
-__global__ void __launch_bounds__(256)
+/*
+ * Second pass of the int8 GMM1 epilogue: whole-row requantisation from the fp32 SwiGLU values. A row is a few KiB, so
+ * one wave takes one row at a time and every lane asks for its (up to eight) 16-byte pieces of the row before it
+ * converts the first. Measured on 131 072 rows of 1536 values (read 805 MB, write 201 MB): 256 threads with one piece
+ * in flight per lane 200 us (5.0 TB/s), two waves with four pieces 182 us, one wave with eight 166 us (6.1 TB/s).
+ */
+constexpr int kRequantThreads = 64, kRequantPieces = 8;
+
+__global__ void __launch_bounds__(kRequantThreads)
 requant_rows_kernel(const float *__restrict__ sgl, const uint32_t *__restrict__ rowmax, const int32_t *__restrict__ row_off,
                     int experts, int I, int8_t *__restrict__ q2, float *__restrict__ scale2)
 {
     const int total = row_off[experts];
+    const int vecs = I / 4;
     for (int row = blockIdx.x; row < total; row += gridDim.x) {
         const float mx = __uint_as_float(rowmax[row]);
         const float inv = mx == 0.0f ? 0.0f : 1.0f / mx;
         if (threadIdx.x == 0) scale2[row] = mx * (1.0f / 127.0f);
-        for (int c = threadIdx.x; c < I / 4; c += blockDim.x) {
-            const f32x4 v = *reinterpret_cast<const f32x4 *>(sgl + (int64_t)row * I + c * 4);
-            uint32_t w = 0;
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(sgl + (int64_t)row * I);
+        uint32_t *dst = reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I);
+        for (int c0 = 0; c0 < vecs; c0 += kRequantThreads * kRequantPieces) {
+            f32x4 v[kRequantPieces];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) w |= ((uint32_t)zb_rint_i8((v[i] * 127.0f) * inv) & 0xffu) << (8 * i);
-            *reinterpret_cast<uint32_t *>(q2 + (int64_t)row * I + c * 4) = w;
+            for (int u = 0; u < kRequantPieces; ++u) {
+                const int c = c0 + u * kRequantThreads + (int)threadIdx.x;
+                v[u] = c < vecs ? __builtin_nontemporal_load(src + c) : f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+            }
+#pragma unroll
+            for (int u = 0; u < kRequantPieces; ++u) {
+                const int c = c0 + u * kRequantThreads + (int)threadIdx.x;
+                uint32_t w = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) w |= ((uint32_t)zb_rint_i8((v[u][i] * 127.0f) * inv) & 0xffu) << (8 * i);
+                if (c < vecs) dst[c] = w;
+            }
         }
     }
 }
@@ -1249,8 +1268,8 @@ extern "C" int32_t zbalhip_gmm1_swiglu_quant(const void *a, const float *a_scale
         const int32_t rc = launch_dma<MODE_W4A8, true, ZDT_BF16>(p, n_tiles, st);
         if (rc != ZBALHIP_OK) return rc;
     }
-    int64_t rb = max_rows < 4096 ? max_rows : 4096;
-    requant_rows_kernel<<<(unsigned)rb, 256, 0, st>>>(sgl_ws, p.rowmax, row_off, (int)experts, (int)(n1 / 2),
+    int64_t rb = max_rows < 16384 ? max_rows : 16384;
+    requant_rows_kernel<<<(unsigned)rb, kRequantThreads, 0, st>>>(sgl_ws, p.rowmax, row_off, (int)experts, (int)(n1 / 2),
                                                     (int8_t *)q2, scale2);
     return zbalhip_check_launch();
 }
