@@ -245,6 +245,48 @@ def test_low_latency_dispatch_at_the_layout_switch(buf, T, H, K, E, mode):
     assert np.array_equal(host(scales).view(np.uint32).reshape(rows, -1)[:total], r_sc.view(np.uint32).reshape(rows, -1)[:total])
 
 
+@pytest.mark.parametrize("T,H,K,E", [
+    (512, 256, 8, 32),       # 4096 picks: the permute kernel works the layout out itself
+    (513, 256, 8, 32),       # one token more: range-layout launch + table in the permute kernel
+    (5000, 128, 8, 32),      # 50 ranges of 100 tokens: the most ranges
+    (3000, 128, 6, 256),     # the most experts the table mode takes (8 ranges of 256 entries)
+    (3000, 128, 6, 257),     # one more: the one-launch layout in front of the permute
+    (200, 128, 32, 64),      # the most picks per token the table mode takes
+    (200, 128, 33, 64),      # one more
+    (4200, 128, 1, 3),       # top-1 on three experts: 1400 rows per expert from 42 ranges
+])
+@pytest.mark.parametrize("qmode", [1, 2])
+def test_fused_permute_quant_layout_modes(buf, T, H, K, E, qmode):
+    """The fused operator's first stage through the kernel ABI, either side of every limit that selects how the layout
+    is derived: rows, scales, ranks, counts and offsets against the oracle, bit for bit, with invalid picks and an
+    expert without rows."""
+    x = bf16_normal((T, H), 71)
+    idx = distinct_topk(T, E, K, 72).astype(np.int32)
+    if E > 3:
+        idx[idx == 1] = 0 if K == 1 else -1           # expert 1 stays empty
+    idx[T // 2, 0] = -1
+    idx[T - 1, K - 1] = E + 7
+    rows = T * K
+    q1 = torch.zeros((rows, H), dtype=torch.uint8, device="cuda")
+    xs = torch.zeros((rows, H // 128 if qmode == 2 else 1), dtype=torch.float32, device="cuda")
+    eidx = torch.full((T, K), -7, dtype=torch.int32, device="cuda")
+    counts = torch.full((E,), -7, dtype=torch.int64, device="cuda")
+    row_off = torch.full((E + 1,), -7, dtype=torch.int32, device="cuda")
+    scratch = torch.zeros((50 * E,), dtype=torch.int32, device="cuda")
+    xd, idd = dev(x), dev(idx)
+    rc = buf.lib.zbalhip_fused_permute_quant(xd.data_ptr(), capi.DT_BF16, idd.data_ptr(), None, None, T, H, K, E, qmode,
+                                             q1.data_ptr(), xs.data_ptr(), eidx.data_ptr(), counts.data_ptr(), row_off.data_ptr(),
+                                             None, 0, scratch.data_ptr(), 50, capi.stream_ptr())
+    capi.check("fused_permute_quant", rc)
+    r_q1, r_xs, r_eidx, r_counts = zo.fused_permute_quant(x, zo.DT_BF16, idx, None, E, qmode)
+    total = int(r_counts.sum())
+    assert np.array_equal(host(counts), r_counts)
+    assert np.array_equal(host(row_off), np.concatenate([[0], np.cumsum(r_counts)]).astype(np.int32))
+    assert np.array_equal(host(eidx), r_eidx)
+    assert np.array_equal(host(q1)[:total], r_q1.view(np.uint8)[:total])
+    assert np.array_equal(host(xs).view(np.uint32).reshape(rows, -1)[:total], r_xs.view(np.uint32).reshape(total, -1))
+
+
 def test_low_latency_token_nums_type_prefix_sum(buf, monkeypatch):
     monkeypatch.setenv("MOE_EXPERT_TOKEN_NUMS_TYPE", "0")
     T, H, K, E = 64, 256, 4, 16
