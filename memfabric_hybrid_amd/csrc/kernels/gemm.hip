@@ -607,7 +607,7 @@ grouped_gemm_dma_kernel(GemmParams p)
     };
 
     /*
-     * DMA: this wave fills 1 KiB blocks wave + NW*j of the A tile (j < 4) and of the W tile (j < W_PARTS). An A block is
+     * DMA: this wave fills 1 KiB blocks wave + NW*j of the A tile (j < A_PARTS) and of the W tile (j < W_PARTS). An A block is
      * tile rows 8*NW*j + r0 with r0 = 8*wave + lane/8, one swizzled 16-byte chunk per lane; rows past the expert's end
      * are clamped onto its last row. 1 KiB block number b = wave + NW*j of the W tile is block b % HALF_BLOCKS of
      * the weight half b / HALF_BLOCKS, a straight copy. Addresses are a wave-uniform base plus a 32-bit lane offset.
@@ -624,7 +624,7 @@ grouped_gemm_dma_kernel(GemmParams p)
      * across the loop they were spilled, and a reload waits for the slabs in flight).
      */
     int lane_dma = lane;
-    /* part j of a slab: the wave's j-th block of the W tile (j < W_PARTS), of the A tile (j < 4) and, with part 0, the scales */
+    /* part j of a slab: the wave's j-th block of the W tile (j < W_PARTS), of the A tile (j < A_PARTS) and, with part 0, the scales */
     auto issue_part = [&](const Tile &t, int kb, int stage, int j) __attribute__((always_inline)) {
         const int lane_x = TM > 256 ? lane_dma : lane;
         const int r0 = 8 * wave_u + (lane_x >> 3);
@@ -749,7 +749,7 @@ grouped_gemm_dma_kernel(GemmParams p)
                 acci[mt][nt] = i32x4{0, 0, 0, 0};
             }
         /*
-         * The wave's 16-row sub-tiles are rows (RG*mt + wm)*16 .. +15 of the tile, mt = 0..3. Only the first `mt_act` of
+         * The wave's 16-row sub-tiles are rows (RG*mt + wm)*16 .. +15 of the tile, mt = 0 .. MTM-1. Only the first `mt_act` of
          * them hold rows of this tile; a wave with none still moves data and meets the barriers, but skips the math.
          */
         const int tile_subs = (cur.row_end - cur.row_begin + 15) >> 4;
