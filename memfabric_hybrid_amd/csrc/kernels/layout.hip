@@ -676,6 +676,7 @@ extern "C" int32_t zbalhip_topk_route(const float *logits, int64_t tokens, int64
     const dim3 grid((unsigned)blocks), block(wpb * 64);
     hipStream_t st = (hipStream_t)stream;
     if (experts <= 64) topk_route_small_kernel<<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
+    else if (experts <= 128) topk_route_kernel<2><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     else if (experts <= 256) topk_route_kernel<4><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     else topk_route_kernel<ZB_MAX_EXPERTS / 64><<<grid, block, 0, st>>>(logits, (int)tokens, (int)experts, (int)topk, topk_idx, idx_is_i64, topk_w);
     return zbalhip_check_launch();
