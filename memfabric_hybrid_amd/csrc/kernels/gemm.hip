@@ -267,9 +267,9 @@ __device__ __forceinline__ void epilogue(const GemmParams &p, const TileCoord &t
  * pairs, so the read is free of bank conflicts whether the LDS serves 8 or 16 lanes per pass; plain
  * row-major storage would put all 16 rows on the same slot.
  *
- * Three shapes are built. TM = 256 and TM = 288 with two stages of 64 / 68 KiB (the slab for step k+1 is in
- * flight while step k is multiplied) have the arithmetic intensity that many-row experts need; the 288-row
- * shape gives the waves of two row groups a fifth sub-tile. TM = 128 with three stages of 48 KiB is for
+ * Three shapes are built. TM = 256 and TM = 320 with two stages of 64 / 72 KiB (the slab for step k+1 is in
+ * flight while step k is multiplied) have the arithmetic intensity that many-row experts need; the 320-row
+ * shape gives every wave a fifth sub-tile. TM = 128 with three stages of 48 KiB is for
  * few-row experts, where the job is to stream every weight byte once at HBM speed: it keeps two weight slabs
  * (64 KiB) in flight per CU, two sub-tiles per wave, and skips the MFMAs of sub-tiles past the expert's end.
  * Either way there is one barrier per step.
@@ -286,14 +286,15 @@ constexpr int D_MAX_EXPERTS = 1024;
 template <int TM, int NSTAGE, int WRB>
 struct DmaShape {
     static constexpr int ROW_GROUPS = 4;                   /* row groups of two waves each: eight waves, two per SIMD */
-    static constexpr int MTM = (TM / 16 + ROW_GROUPS - 1) / ROW_GROUPS;   /* 16-row sub-tiles per wave, at most: 4, or 5 in the 288-row shape */
+    static constexpr int MTM = (TM / 16 + ROW_GROUPS - 1) / ROW_GROUPS;   /* 16-row sub-tiles per wave, at most: 2, 4, or 5 in the 320-row shape */
     static constexpr int NW = ROW_GROUPS * 2;
     static constexpr int THREADS = NW * 64;
     static constexpr int A_BYTES = TM * BKB;
     static constexpr int W_BYTES = BN * WRB;
     static constexpr int STAGE_BYTES = A_BYTES + W_BYTES;
     static constexpr int HALF_BLOCKS = 128 * WRB / 1024;   /* 1 KiB blocks per 128-channel half: 16 or 8 */
-    static constexpr int A_PARTS = (A_BYTES / 1024 + NW - 1) / NW;   /* 1 KiB blocks of the A tile per wave: 4 (288 rows: 5, the last for half of the waves) */
+    static constexpr int MAX_EXPERTS = TM > 256 ? 512 : D_MAX_EXPERTS;   /* what the lookup tables hold: the 320-row shape has 160 KiB of LDS less 144 KiB of stages for everything else */
+    static constexpr int A_PARTS = (A_BYTES / 1024 + NW - 1) / NW;   /* 1 KiB blocks of the A tile per wave: 2, 4 or 5 */
     static constexpr int W_PARTS = W_BYTES / 1024 / NW;    /* 1 KiB blocks of the W tile per wave (2, 4 or 8) */
     static constexpr int PARTS = W_PARTS > A_PARTS ? W_PARTS : A_PARTS;
     static constexpr bool TWO_PHASE = TM == 256;            /* the tiles of short experts run after all the others (see the kernel) */
@@ -302,8 +303,8 @@ struct DmaShape {
     static constexpr int SW_BYTES = 2 * SW_STRIDE * 4;
     static_assert(SW_STRIDE >= 2 * D_MAX_KB && SW_STRIDE >= 256 + TM, "scale buffer too small");
     static constexpr int LDS_BYTES = NSTAGE * STAGE_BYTES + NSTAGE * TM * 4 + 2 * TM * 4 + SW_BYTES +
-                                     2 * (D_MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0) +
-                                     (TWO_PHASE ? D_MAX_EXPERTS * 2 + (D_MAX_EXPERTS + 1) * 4 : 0);
+                                     2 * (MAX_EXPERTS + 1) * 4 + (WRB == 64 ? NSTAGE * BN * 2 : 0) +
+                                     (TWO_PHASE ? MAX_EXPERTS * 2 + (MAX_EXPERTS + 1) * 4 : 0);
     static_assert(PARTS >= 2 && (PARTS % 4 == 0 || PARTS == 2 || (NSTAGE == 2 && PARTS == 5)),
                   "the issue schedule hands out parts q * PARTS / 4 .. (q + 1) * PARTS / 4 - 1 of a slab with quarter q of a step");
     static_assert(NW <= HALF_BLOCKS && HALF_BLOCKS % NW == 0, "a wave's W blocks must not straddle a weight half");
@@ -408,10 +409,10 @@ grouped_gemm_dma_kernel(GemmParams p)
     constexpr int SW_STRIDE = S::SW_STRIDE;
     float *lds_sw = lds_rowmax + 2 * TM;                                      /* [2 tiles][SW_STRIDE]: fp8 [2][D_MAX_KB] weight block scales */
     int *lds_mtp = reinterpret_cast<int *>(lds_sw + 2 * SW_STRIDE);            /* [experts + 1] tiles of TM rows before expert e */
-    int *lds_roff = lds_mtp + (D_MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
-    uint16_t *lds_gs = reinterpret_cast<uint16_t *>(lds_roff + (D_MAX_EXPERTS + 1));   /* [NSTAGE][BN] W4A8 group scales (fp16) */
+    int *lds_roff = lds_mtp + (S::MAX_EXPERTS + 1);                            /* [experts + 1] copy of row_off */
+    uint16_t *lds_gs = reinterpret_cast<uint16_t *>(lds_roff + (S::MAX_EXPERTS + 1));   /* [NSTAGE][BN] W4A8 group scales (fp16) */
     uint16_t *lds_short = lds_gs + (WRB == 64 ? NSTAGE * BN : 0);                       /* [experts] the short experts, second phase */
-    int *lds_cost = reinterpret_cast<int *>(lds_short + D_MAX_EXPERTS);                 /* [experts + 1] 16-row sub-tiles of the main tiles before expert e */
+    int *lds_cost = reinterpret_cast<int *>(lds_short + S::MAX_EXPERTS);                 /* [experts + 1] 16-row sub-tiles of the main tiles before expert e */
     constexpr bool TWO_PHASE = S::TWO_PHASE;
 
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -619,7 +620,7 @@ grouped_gemm_dma_kernel(GemmParams p)
     const bool gs_wave = MODE == MODE_W4A8 && wave < 2;            /* wave h brings the group scales of weight half h */
     const uint32_t lds_gs0 = __builtin_amdgcn_readfirstlane(lds_addr(lds_gs) + (wave & 1) * 256);
     /*
-     * The 288-row shape has no register to spare for the transfers' lane offsets across a K step: there they are worked
+     * The 320-row shape has no register to spare for the transfers' lane offsets across a K step: there they are worked
      * out afresh for every transfer from a copy of the lane number that the K loop makes opaque once per step (kept
      * across the loop they were spilled, and a reload waits for the slabs in flight).
      */
@@ -1166,7 +1167,7 @@ int32_t prepare_mode()
     int n = 0;
     int32_t rc = prepare_shape<MODE, GMM1, OUT_DT, 256, 2, false>(nullptr, &n);
     if constexpr (MODE != MODE_W4A8)
-        if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 288, 2, false>(nullptr, &n);
+        if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 320, 2, false>(nullptr, &n);
     if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 128, 3, false>(nullptr, &n);
     if constexpr (MODE != MODE_W4A8)
         if (rc == ZBALHIP_OK) rc = prepare_shape<MODE, GMM1, OUT_DT, 128, 3, true>(nullptr, &n);
@@ -1176,9 +1177,9 @@ int32_t prepare_mode()
 /*
  * Shape choice from what the host knows (the row counts themselves live on the device). With few rows per expert the
  * GEMM is a weight-streaming job and takes the three-stage 128-row shape (which needs two K slabs to fill its
- * pipeline); with many it needs the arithmetic intensity of a two-stage shape, 288 or 256 rows high. The shapes were
+ * pipeline); with many it needs the arithmetic intensity of a two-stage shape, 320 or 256 rows high. The shapes were
  * timed against each other on 7168 x 4096 / 2048 x 7168 experts (W4A8: 4096 x 3072 / 1536 x 4096, 128 experts) with 32
- * and with 256 experts, random routing; rows per expert on average, first / second GEMM, 128-row against 288-row
+ * and with 256 experts, random routing; rows per expert on average, first / second GEMM, 128-row against tall
  * (W4A8: 256-row) shape in ms:
  *   - fp8, 32 experts: 128 rows 0.247 / 0.136 against 0.256 / 0.145; 192 rows 0.298 / 0.160 against 0.278 / 0.166;
  *     256 rows 0.369 / 0.194 against 0.306 / 0.188. 256 experts: 128 rows 1.889 / 0.961 against 1.877 / 1.088;
@@ -1200,15 +1201,21 @@ inline int64_t few_rows_limit(const GemmParams &p, int n_tiles)
 /*
  * Two thirds of a two-stage tile's time does not depend on its rows (weight fragments, barrier, slab transfers), so
  * the fewer row tiles an expert has the better, and an expert whose rows just miss a multiple of 256 pays for a whole
- * tile more. The 288-row shape cuts an expert into ceil(rows / 288) even tiles: where that is as many as
- * ceil(rows / 256) they are the same tiles as the 256-row shape's (and cost 1-4 % more in this kernel), where it is one
- * less the expert is a tile's fixed cost shorter. Under random routing the second case is common as long as an expert
- * has few tiles. Measured against the 256-row shape, first / second GEMM, rows per expert on average: fp8 256 rows
- * -29 % / -15 %, 512 rows -16 % / -9 %, 1024 rows -7.6 % / -4.7 %, 1500 rows -2 % / +1.4 %, 2048 rows +0.5 % / +2 %;
- * W8A8 256 rows -26 % / -17 %, 1024 rows -7 % / -7 %; with exactly 1024 rows for every expert fp8 +3 % / +4.6 %.
- * W4A8 has no such shape (its loop has no registers for a fifth row sub-tile).
+ * tile more. The tall shape (five sub-tiles per wave; first built 288 rows high, then 320, which is the same loop and
+ * 1.5 % faster even on the same tiles) cuts an expert into ceil(rows / 320) even tiles: where that is as many as
+ * ceil(rows / 256) they are the same tiles as the 256-row shape's (and cost 1-4 % more in this kernel), where it is
+ * fewer the expert is a tile's fixed cost shorter. Measured against the 256-row shape on 32 experts of 7168 x 4096 /
+ * 2048 x 7168, random routing, first / second GEMM, rows per expert on average:
+ *   - fp8: 256 rows -29 % / -15 %, 512 rows -16 % / -9 %, 1024 rows -8 % / -5 % (the 288-row build; 320 rows another
+ *     -2 % / 0 %), 1500 rows 0 / +3 %, 2048 rows +2 % / +2 %, 3072 rows +2 % / +4 %, 4096 rows +2 % / +3 %: its
+ *     five-sub-tile loop goes over the weight fragments twice and gives back what the saved tiles bring, hence the limit;
+ *   - W8A8: 256 rows -26 % / -17 %, 1024 rows -9 % / -5 %, 1500 rows -5 % / -5 %, 2048 rows -4.5 % / -8 %, 3072 rows
+ *     -3 % / -6 %, 4096 rows -5 % / -9 %: no limit;
+ *   - with exactly 1024 rows for every expert fp8 +3 % / +4.6 % (the 288-row build).
+ * W4A8 has no such shape (its loop has no registers for a fifth row sub-tile). The tall shape's LDS leaves room for
+ * lookup tables of 512 experts; launches with more take the 256-row shape.
  */
-constexpr int64_t kTallRowsLimit = 1536;
+constexpr int64_t kTallRowsLimitFp8 = 1536;
 
 template <int MODE, bool GMM1, int OUT_DT>
 int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
@@ -1229,7 +1236,9 @@ int32_t launch_dma(const GemmParams &p, int n_tiles, hipStream_t st)
         return launch_dma_shape<MODE, GMM1, OUT_DT, 128, 3>(p, n_tiles, st);
     }
     if constexpr (MODE != MODE_W4A8) {
-        if ((int64_t)p.max_rows <= kTallRowsLimit * (int64_t)p.experts) return launch_dma_shape<MODE, GMM1, OUT_DT, 288, 2>(p, n_tiles, st);
+        using Tall = DmaShape<320, 2, 128>;
+        const bool tall_pays = MODE == MODE_W8A8 || (int64_t)p.max_rows <= kTallRowsLimitFp8 * (int64_t)p.experts;
+        if (tall_pays && p.experts <= Tall::MAX_EXPERTS) return launch_dma_shape<MODE, GMM1, OUT_DT, 320, 2>(p, n_tiles, st);
     }
     return launch_dma_shape<MODE, GMM1, OUT_DT, 256, 2>(p, n_tiles, st);
 }

@@ -109,21 +109,21 @@ def test_gmm1_w8a8_bit_exact(buf, E, K, N1, rows):
     assert np.array_equal(host(q2), r_q2)
 
 
-# experts with no rows, with only a short tile, with exactly full tiles of either two-stage shape (256 and 288 rows), one
-# row more than those, 17 and 18 sub-tiles of 16 rows (five per wave in some or all row groups of the 288-row shape), and
-# with short tails of both classes (up to a quarter and up to half of a tile): the two-stage shapes run the short tails
+# experts with no rows, with only a short tile, with exactly full tiles of either two-stage shape (256 and 320 rows), one
+# row more than those, 17 to 20 sub-tiles of 16 rows (five per wave in some or all row groups of the 320-row shape), and
+# with short tails of both classes (up to a quarter and up to half of a tile): the 256-row shape runs the short tails
 # after all other tiles, the longer class first
-TILE_ORDER_COUNTS = np.array([0, 5, 256, 257, 300, 320, 384, 385, 1024, 1030, 130, 64, 0, 512 + 128, 511, 1, 288, 289, 273, 576],
-                             dtype=np.int64)
+TILE_ORDER_COUNTS = np.array([0, 5, 256, 257, 300, 320, 321, 384, 385, 1024, 1030, 130, 64, 0, 512 + 128, 511, 1, 288, 289, 273,
+                              576, 305, 641], dtype=np.int64)
 
 
 @pytest.mark.parametrize("N", [256, 1280])
-@pytest.mark.parametrize("big", [2048, 40000])           # rows of one expert: the average selects the 288-row / the 256-row shape
+@pytest.mark.parametrize("big", [2048, 40000])           # rows of one expert: a few tiles, or more than a hundred
 def test_gemms_w8a8_tile_order_with_short_tails_bit_exact(buf, N, big):
     counts, K = TILE_ORDER_COUNTS.copy(), 384
-    counts[8] = big
+    counts[9] = big
     E, rows = len(counts), int(counts.sum())
-    assert (192 * E < rows <= 1536 * E) if big == 2048 else (rows > 1536 * E)
+    assert rows > 192 * E                                     # beyond the few-row shape: W8A8 takes the 320-row shape
     a = rng(61).integers(-127, 128, (rows, K)).astype(np.int8)
     xs = rng(62).uniform(0.005, 0.05, rows).astype(np.float32)
     w = rng(63).integers(-16, 16, (E, K, N)).astype(np.int8)
@@ -136,12 +136,12 @@ def test_gemms_w8a8_tile_order_with_short_tails_bit_exact(buf, N, big):
     assert np.array_equal(host(q2), r_q2)
 
 
-@pytest.mark.parametrize("big", [1024, 40000])           # as above
+@pytest.mark.parametrize("big", [1024, 40000])           # rows of one expert: the average selects the 320-row / the 256-row shape
 def test_gemms_fp8_tile_order_with_short_tails(buf, big):
     counts, K, N = TILE_ORDER_COUNTS.copy(), 256, 512
-    counts[8] = big
+    counts[9] = big
     E, rows = len(counts), int(counts.sum())
-    assert (96 * E < rows <= 1536 * E) if big == 1024 else (rows > 1536 * E)
+    assert (128 * E < rows <= 1536 * E) if big == 1024 else (rows > 1536 * E)
     a, sa, w, sw = fp8_operands(E, K, N, rows, 70)
     y = gmm2(buf, dev(a), dev(sa), buf.prepack_weight(dev(w)), dev(sw), capi.DT_FP32, counts, K, N, 2)
     ref = zo.gmm2_fp8(a, sa, w, sw, counts)
@@ -172,7 +172,7 @@ def test_gemms_w8a8_even_row_tiles_in_the_few_row_shape_bit_exact(buf):
     assert np.array_equal(host(q2), r_q2)
 
 
-@pytest.mark.parametrize("rows", [40000, 200000])      # few rows per expert (128-row shape) / many (288-row shape)
+@pytest.mark.parametrize("rows", [40000, 200000])      # few rows per expert (128-row shape) / many (256-row shape: more experts than the 320-row shape's tables hold)
 def test_gmm2_w8a8_largest_expert_count_bit_exact(buf, rows):
     """1024 experts, the most the kernel's lookup tables hold: the tile lookup, the cost prefix and the list of short
     experts all run over sixteen 64-expert chunks. Skewed counts leave many experts empty or short."""
@@ -239,9 +239,9 @@ def test_gmm1_fp8(buf, E, K, N1, rows):
 
 @pytest.mark.parametrize("rows_per_expert", [96, 97, 128, 129, 192, 193, 1536, 1537])
 def test_gemms_at_the_shape_limits(buf, rows_per_expert):
-    """The launcher picks the 128-row, the 288-row or the 256-row shape from rows / experts (few rows: up to 64 .. 192
-    by mode and GEMM; 288-row tiles up to 1536): the same operands either side of every limit, W8A8 bit exact and fp8
-    within its tolerance."""
+    """The launcher picks the 128-row, the 320-row or the 256-row shape from rows / experts (few rows: up to 96 .. 192
+    by mode and GEMM; fp8 takes 320-row tiles up to 1536 rows): the same operands either side of every limit, W8A8
+    bit exact and fp8 within its tolerance."""
     E, K, N = 4, 256, 512
     rows = rows_per_expert * E
     counts = ragged_counts(E, rows, 7 * rows_per_expert)
@@ -268,7 +268,7 @@ def test_gemms_at_the_shape_limits(buf, rows_per_expert):
 
 # ---- both workgroup shapes, with more tiles than workgroups ------------------------------------------------------
 
-@pytest.mark.parametrize("E,K,N,rows", [(8, 256, 2304, 8192),     # 1024 rows per expert: 288-row tiles, 2 stages, ~300 tiles
+@pytest.mark.parametrize("E,K,N,rows", [(8, 256, 2304, 8192),     # 1024 rows per expert: 320-row tiles, 2 stages, ~300 tiles
                                         (64, 256, 1024, 8000),    # <= 128 on average: 128-row tiles, 3 stages, ~400 tiles
                                         (4, 128, 256, 3000)])     # a single K slab
 def test_gmm2_w8a8_many_tiles_per_workgroup(buf, E, K, N, rows):
@@ -763,8 +763,8 @@ def test_w8a8_gemms_random_row_counts_bit_exact(buf, seed):
             hot = r.choice(E, size=min(E, 3), replace=False)
             counts[hot] = r.integers(1, 1500, size=len(hot))
         elif style == 2:
-            counts = r.choice([0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 271, 272, 273, 287, 288, 289, 383, 384,
-                               385, 513, 575, 576, 577], size=E)
+            counts = r.choice([0, 1, 15, 16, 17, 63, 64, 65, 127, 128, 129, 255, 256, 257, 271, 272, 273, 287, 288, 289, 319, 320,
+                               321, 383, 384, 385, 513, 575, 576, 577, 639, 640, 641], size=E)
             if counts.sum() > 6000:
                 counts = counts // 4
         else:
